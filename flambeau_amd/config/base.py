@@ -67,6 +67,22 @@ class KeyReader:
             raise ConfigError(f"{self.where}: key '{key}' must be true or false, got {v!r}")
         return v
 
+    def section(self, key: str, default: Any = _MISSING):
+        """A nested object as a reader of its own (errors name the path), or ``default``."""
+        v = self._get(key, default)
+        if v is _MISSING:
+            return default
+        if not isinstance(v, dict):
+            raise ConfigError(f"{self.where}: key '{key}' must be an object, got {v!r}")
+        return KeyReader(v, f"{self.where}: {key}")
+
+    def sections(self, key: str):
+        """A list of objects, each as a reader."""
+        v = self._get(key, _MISSING)
+        if not isinstance(v, list) or not all(isinstance(x, dict) for x in v):
+            raise ConfigError(f"{self.where}: key '{key}' must be a list of objects")
+        return [KeyReader(x, f"{self.where}: {key}[{i}]") for i, x in enumerate(v)]
+
     def string(self, key: str, default: Any = _MISSING):
         v = self._get(key, default)
         if v is _MISSING:
@@ -90,8 +106,11 @@ def read_config_json(model_dir) -> dict:
 
 
 def architecture_name(raw: dict, where: str = "config.json") -> str:
-    """``architectures[0]``: the name the registry is asked for."""
+    """``architectures[0]``, or the string under ``architecture``: the name the registry is asked for."""
     archs = raw.get("architectures")
-    if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
-        raise ConfigError(f"{where}: missing key 'architectures' (a list with the model class name)")
-    return archs[0]
+    if isinstance(archs, list) and archs and isinstance(archs[0], str):
+        return archs[0]
+    one = raw.get("architecture")
+    if isinstance(one, str) and one:
+        return one
+    raise ConfigError(f"{where}: missing key 'architectures' (a list with the model class name) or 'architecture' (its name)")

@@ -60,6 +60,45 @@ int fl_sample_bias(float* logits, int V, int n, const float* row, const float* t
 int fl_sample_count(unsigned short* counts, int V, int rows, const float* slot, const int* ids, hipStream_t stream);
 int fl_sample_history(unsigned short* counts, int V, int slot, const int* tokens, int n, hipStream_t stream);
 
+// ---- attention over one cached latent per token (latent.hip) ----
+// RMS norm of columns col0 .. col0 + width - 1 of float rows; with a block table the result goes to the
+// page row of the token's position (pool [n_pages][page_size][width]), else to out [n][width]
+int fl_norm_slice(const float* x, int ld, int col0, int width, const float* w, float eps, void* out,
+                  int out_dtype, int n, const int* positions, const int* tok_seq, const int* block_table,
+                  int max_blocks, int page_size, int n_pages, hipStream_t stream);
+// one small product per head: out[t][h][:] = x[t][h][:] W_h (transposed: W_h^T), optionally times the sigmoid of a gate logit per head
+int fl_heads_matmul(const float* x, int ldx, const void* w, int w_dtype, void* out, int out_dtype, int n,
+                    int H, int K, int J, int transposed, const float* gate, int ldg, int gate_col0,
+                    hipStream_t stream);
+// z[t][h][:] = softmax_j(scale * qa[t][h] . c_j) c_j over the latent rows j <= position of the token's request
+int fl_latent_attention(const float* qa, float* z, const void* pool, int dtype, const int* positions,
+                        const int* tok_seq, const int* block_table, int max_blocks, int n, int H, int R,
+                        int page_size, int n_pages, float scale, int window, hipStream_t stream);
+int fl_latent_max_width(void);
+
+// ---- the mLSTM recurrence (mlstm.hip) ----
+int fl_mlstm_scan(const float* proj, int ld, int col_q, int col_k, int col_v, int col_i, int col_f,
+                  const float* bias_i, const float* bias_f, float cap, float q_scale, float* state,
+                  const int* seq_q_start, const int* seq_q_len, const int* seq_slots, float* out,
+                  int n_seqs, int H, int D, int Dv, hipStream_t stream);
+int fl_mlstm_max_dim(void);
+long fl_mlstm_state_floats(int D, int Dv);
+int fl_headnorm_gate(const float* x, const float* w, const float* gate, int ldg, int gate_col0, void* out,
+                     int out_dtype, int n, int H, int Dv, float eps, hipStream_t stream);
+
+// ---- routed experts, activations, re-entry of the stream (moe.hip) ----
+int fl_moe_route(const float* logits, int ld, int col0, int n, int E, int top, int kind, int renorm,
+                 int* place, int* src_row, float* src_scale, float* pair_w, int* tiles, int max_tiles,
+                 hipStream_t stream);
+int fl_moe_tile_rows(void);
+int fl_moe_gemm(const void* x, int dtype, const int* src_row, const float* src_scale, const void* w,
+                float* out, const int* tiles, int max_tiles, int N, int K, hipStream_t stream);
+int fl_moe_combine(const float* y, const int* place, int top, const float* shared, const float* gate, int ldg,
+                   int gate_col, float* delta, int n, int W, hipStream_t stream);
+int fl_activation(const float* x, void* out, int out_dtype, long total, int kind, hipStream_t stream);
+int fl_concat_cast(const float* a, const float* b, void* out, int out_dtype, int n, int W, hipStream_t stream);
+int fl_add_rowvec(float* x, const float* v, int n, int W, hipStream_t stream);
+
 // ---- tuned bf16 kernels ----
 // nw_hint: waves per block that split K (0: chosen from the sizes)
 // epilogue: 0 = plain product; 1 = SwiGLU over interleaved gate/up rows, out_cols <= N / 2

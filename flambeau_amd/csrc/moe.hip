@@ -1,0 +1,302 @@
+// A feed-forward of routed experts: the router's choice, the experts' products over the rows each
+// was given, and the sum per token.
+//
+//   fl_moe_route    scores -> for every token its `top` experts (largest router logits, the lower index among
+//                   equals) and their weights; the (token, expert) pairs sorted by expert, cut into row
+//                   tiles that each belong to one expert
+//   fl_moe_gemm     out[p] = (scale[p] * x[src[p]]) W_e^T for the sorted pairs p, e the expert of p's tile
+//   fl_moe_combine  delta[t] = sum_k y[place of (t, k)]  (+ sigmoid(shared gate logit) * shared[t])
+// Nothing of a step's values is read on the host: the lists live on the device and the grids are
+// sized by their upper bounds (tiles that a step does not use end at once).
+#include "common.h"
+#include "api.h"
+#include "recordable.h"
+
+#define MOE_TILE 64           // rows of a tile of fl_moe_gemm
+#define MOE_MAX_EXPERTS 1024
+#define MOE_MAX_TOP 16
+
+// logits: float rows ld wide, the experts' at col0 .. col0 + E - 1.  kind 0: weight = sigmoid(logit);
+// kind 1: weight = softmax over all experts.  renorm: the chosen weights are divided by their sum.
+// place [n * top]: where pair (t, k) lies in the sorted order; src_row / src_scale [n * top]: token and weight
+// of every sorted place; tiles [max_tiles][4] = (expert, first place, places, 0), expert -1: unused.
+__global__ __launch_bounds__(1024) void moe_route_kernel(const float* __restrict__ logits, int ld, int col0, int n, int E,
+                                                         int top, int kind, int renorm, int* __restrict__ place,
+                                                         int* __restrict__ src_row, float* __restrict__ src_scale,
+                                                         float* __restrict__ pair_w, int* __restrict__ tiles, int max_tiles) {
+    __shared__ int count[MOE_MAX_EXPERTS];
+    __shared__ int first[MOE_MAX_EXPERTS];
+    for (int e = threadIdx.x; e < E; e += 1024) count[e] = 0;
+    __syncthreads();
+    for (int t = threadIdx.x; t < n; t += 1024) {
+        const float* z = logits + (size_t)t * ld + col0;
+        float zmax = -INFINITY, zsum = 0.f;
+        if (kind == 1) {
+            for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, z[e]);
+            for (int e = 0; e < E; ++e) zsum += expf(z[e] - zmax);
+        }
+        int chosen[MOE_MAX_TOP];
+        float w[MOE_MAX_TOP], wsum = 0.f;
+        for (int k = 0; k < top; ++k) {
+            int best = -1;
+            float bz = -INFINITY;
+            for (int e = 0; e < E; ++e) {
+                bool taken = false;
+                for (int u = 0; u < k; ++u) taken |= chosen[u] == e;
+                if (!taken && (best < 0 || z[e] > bz)) { best = e; bz = z[e]; }
+            }
+            chosen[k] = best;
+            w[k] = kind == 1 ? expf(bz - zmax) / zsum : 1.0f / (1.0f + expf(-bz));
+            wsum += w[k];
+        }
+        for (int k = 0; k < top; ++k) {
+            place[(size_t)t * top + k] = chosen[k];
+            pair_w[(size_t)t * top + k] = renorm ? w[k] / wsum : w[k];
+            atomicAdd(&count[chosen[k]], 1);
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0, tile = 0;
+        for (int e = 0; e < E; ++e) {
+            first[e] = at;
+            for (int r = 0; r < count[e] && tile < max_tiles; r += MOE_TILE, ++tile) {
+                tiles[4 * tile + 0] = e;
+                tiles[4 * tile + 1] = at + r;
+                tiles[4 * tile + 2] = min(MOE_TILE, count[e] - r);
+                tiles[4 * tile + 3] = 0;
+            }
+            at += count[e];
+            count[e] = 0;                      // from here on: places handed out
+        }
+        for (; tile < max_tiles; ++tile) {
+            tiles[4 * tile + 0] = -1;
+            tiles[4 * tile + 1] = tiles[4 * tile + 2] = tiles[4 * tile + 3] = 0;
+        }
+    }
+    __syncthreads();
+    // a token's pairs take the next free places of their experts; which of an expert's places a pair
+    // gets changes nothing in its result (every row of the products is computed on its own)
+    for (int a = threadIdx.x; a < n * top; a += 1024) {
+        const int e = place[a];
+        const int p = first[e] + atomicAdd(&count[e], 1);
+        src_row[p] = a / top;
+        src_scale[p] = pair_w[a];
+        place[a] = p;
+    }
+}
+
+extern "C" int fl_moe_tile_rows(void) { return MOE_TILE; }
+
+extern "C" int fl_moe_route(const float* logits, int ld, int col0, int n, int E, int top, int kind, int renorm,
+                            int* place, int* src_row, float* src_scale, float* pair_w, int* tiles, int max_tiles,
+                            hipStream_t stream) {
+    FL_CHECK(n >= 0 && E > 0 && E <= MOE_MAX_EXPERTS && top > 0 && top <= MOE_MAX_TOP && top <= E,
+             "moe_route: %d of %d experts (at most %d of %d)", top, E, MOE_MAX_TOP, MOE_MAX_EXPERTS);
+    FL_CHECK(ld >= col0 + E && col0 >= 0, "moe_route: columns %d..%d of rows %d wide", col0, col0 + E, ld);
+    {
+        const long pairs = (long)n * top;          // an expert's last tile may be short: pairs / 64 full tiles and one per expert at most
+        FL_CHECK((long)max_tiles >= pairs / MOE_TILE + (pairs < E ? pairs : E), "moe_route: %d tiles cannot hold %ld rows of %d experts", max_tiles, pairs, E);
+    }
+    FL_CHECK(kind == 0 || kind == 1, "moe_route: unknown scoring %d", kind);
+    if (n == 0) return 0;
+    moe_route_kernel<<<1, 1024, 0, stream>>>(logits, ld, col0, n, E, top, kind, renorm, place, src_row, src_scale, pair_w, tiles, max_tiles);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_moe_route)
+
+// The plain product (64 x 64 tile, 4 x 4 per thread, k in steps of 16, the steps' sums added with a
+// compensated addition) over the rows of one tile of one expert.  src_row / src_scale may be null (the
+// rows are then the sorted places themselves, unscaled).  A scaled row is rounded to the storage type
+// before it is multiplied, as a stored activation would be.
+template <typename TIn>
+__global__ __launch_bounds__(256) void moe_gemm_kernel(const TIn* __restrict__ x, const int* __restrict__ src_row,
+                                                       const float* __restrict__ src_scale, const TIn* __restrict__ w,
+                                                       float* __restrict__ out, const int* __restrict__ tiles, int N, int K) {
+    __shared__ float xs[16][68];
+    __shared__ float ws[16][68];
+    __shared__ int rows_of[MOE_TILE];
+    __shared__ float scale_of[MOE_TILE];
+    const int e = tiles[4 * blockIdx.y + 0];
+    if (e < 0) return;
+    const int p0 = tiles[4 * blockIdx.y + 1], M = tiles[4 * blockIdx.y + 2];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int n0 = blockIdx.x * 64;
+    const TIn* we = w + (size_t)e * N * K;
+    if (threadIdx.x < MOE_TILE) {
+        const int i = threadIdx.x;
+        rows_of[i] = i < M ? (src_row ? src_row[p0 + i] : p0 + i) : 0;
+        scale_of[i] = (i < M && src_scale) ? src_scale[p0 + i] : 1.0f;
+    }
+    __syncthreads();
+    float acc[4][4], lost[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { acc[i][j] = 0.f; lost[i][j] = 0.f; }
+    for (int k0 = 0; k0 < K; k0 += 16) {
+        for (int el = threadIdx.x; el < 1024; el += 256) {
+            const int row = el >> 4, kk = el & 15;
+            const int gk = k0 + kk, gn = n0 + row;
+            float xv = 0.f;
+            if (row < M && gk < K) {
+                xv = to_f32(x[(size_t)rows_of[row] * K + gk]);
+                if (src_scale) xv = to_f32(from_f32<TIn>(xv * scale_of[row]));
+            }
+            xs[kk][row] = xv;
+            ws[kk][row] = (gn < N && gk < K) ? to_f32(we[(size_t)gn * K + gk]) : 0.f;
+        }
+        __syncthreads();
+        float part[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) part[i][j] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = xs[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = ws[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) part[i][j] = fmaf(a[i], b[j], part[i][j]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float y = part[i][j] - lost[i][j];
+                const float t = acc[i][j] + y;
+                lost[i][j] = (t - acc[i][j]) - y;
+                acc[i][j] = t;
+            }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = ty * 4 + i;
+        if (r >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int gn = n0 + tx * 4 + j;
+            if (gn < N) out[(size_t)(p0 + r) * N + gn] = acc[i][j];
+        }
+    }
+}
+
+extern "C" int fl_moe_gemm(const void* x, int dtype, const int* src_row, const float* src_scale, const void* w,
+                           float* out, const int* tiles, int max_tiles, int N, int K, hipStream_t stream) {
+    FL_CHECK(max_tiles >= 0 && N > 0 && K > 0, "moe_gemm: bad sizes");
+    if (max_tiles == 0) return 0;
+    FL_CHECK(max_tiles <= 65535, "moe_gemm: %d row tiles are more than one grid takes", max_tiles);
+    dim3 grid(ceil_div(N, 64), max_tiles);
+    if (dtype == FL_F32)
+        moe_gemm_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, src_row, src_scale, (const float*)w, out, tiles, N, K);
+    else if (dtype == FL_BF16)
+        moe_gemm_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, src_row, src_scale, (const bf16_t*)w, out, tiles, N, K);
+    else
+        FL_CHECK(false, "moe_gemm: unknown dtype %d", dtype);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_moe_gemm)
+
+// delta[t][c] = sum over k (rising) of y[place[t * top + k]][c], plus sigmoid(gate logit of t) * shared[t][c]
+// where a shared expert is given (gate: float rows ldg wide, the logit at gate_col; null: ungated).
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ place, int top,
+                                                          const float* __restrict__ shared, const float* __restrict__ gate,
+                                                          int ldg, int gate_col, float* __restrict__ delta, int W) {
+    const int t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= W) return;
+    float v = 0.f;
+    for (int k = 0; k < top; ++k) v += y[(size_t)place[(size_t)t * top + k] * W + c];
+    if (shared) {
+        const float g = gate ? 1.0f / (1.0f + expf(-gate[(size_t)t * ldg + gate_col])) : 1.0f;
+        v += g * shared[(size_t)t * W + c];
+    }
+    delta[(size_t)t * W + c] = v;
+}
+
+extern "C" int fl_moe_combine(const float* y, const int* place, int top, const float* shared, const float* gate, int ldg,
+                              int gate_col, float* delta, int n, int W, hipStream_t stream) {
+    FL_CHECK(n >= 0 && W > 0 && top >= 0, "moe_combine: bad sizes");
+    FL_CHECK(!gate || (gate_col >= 0 && ldg > gate_col), "moe_combine: gate column %d of rows %d wide", gate_col, ldg);
+    if (n == 0) return 0;
+    FL_CHECK(n <= 65535, "moe_combine: %d rows are more than one grid takes", n);
+    dim3 grid(ceil_div(W, 256), n);
+    moe_combine_kernel<<<grid, 256, 0, stream>>>(y, place, top, shared, gate, ldg, gate_col, delta, W);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_moe_combine)
+
+// ------------------------------------------------------------------ activations of an ungated feed-forward
+// kind 0: gelu with the error function, 0.5 z (1 + erf(z / sqrt 2)); 1: its tanh form,
+// 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))); 2: silu, z / (1 + exp(-z)).
+template <typename TOut>
+__global__ __launch_bounds__(256) void activation_kernel(const float* __restrict__ x, TOut* __restrict__ out, long total, int kind) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const float z = x[i];
+    float y;
+    if (kind == 0) y = 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f));
+    else if (kind == 1) y = 0.5f * z * (1.0f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
+    else y = z / (1.0f + expf(-z));
+    out[i] = from_f32<TOut>(y);
+}
+
+extern "C" int fl_activation(const float* x, void* out, int out_dtype, long total, int kind, hipStream_t stream) {
+    FL_CHECK(total >= 0 && kind >= 0 && kind <= 2, "activation: bad size or kind %d", kind);
+    if (total == 0) return 0;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    if (out_dtype == FL_F32) activation_kernel<float><<<blocks, 256, 0, stream>>>(x, (float*)out, total, kind);
+    else if (out_dtype == FL_BF16) activation_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, (bf16_t*)out, total, kind);
+    else FL_CHECK(false, "activation: unknown dtype %d", out_dtype);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_activation)
+
+// ------------------------------------------------------------------ re-entry of the residual stream
+// out[r] = [a[r] ; b[r]] in the storage type (two float rows of W values side by side).
+template <typename TOut>
+__global__ __launch_bounds__(256) void concat_cast_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                          TOut* __restrict__ out, int W) {
+    const int r = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= 2 * W) return;
+    out[(size_t)r * 2 * W + c] = from_f32<TOut>(c < W ? a[(size_t)r * W + c] : b[(size_t)r * W + c - W]);
+}
+
+extern "C" int fl_concat_cast(const float* a, const float* b, void* out, int out_dtype, int n, int W, hipStream_t stream) {
+    FL_CHECK(n >= 0 && W > 0, "concat_cast: bad sizes");
+    if (n == 0) return 0;
+    FL_CHECK(n <= 65535, "concat_cast: %d rows are more than one grid takes", n);
+    dim3 grid(ceil_div(2 * W, 256), n);
+    if (out_dtype == FL_F32) concat_cast_kernel<float><<<grid, 256, 0, stream>>>(a, b, (float*)out, W);
+    else if (out_dtype == FL_BF16) concat_cast_kernel<bf16_t><<<grid, 256, 0, stream>>>(a, b, (bf16_t*)out, W);
+    else FL_CHECK(false, "concat_cast: unknown dtype %d", out_dtype);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_concat_cast)
+
+// x[r][c] += v[c]
+__global__ __launch_bounds__(256) void add_rowvec_kernel(float* __restrict__ x, const float* __restrict__ v, int W) {
+    const int r = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    if (c < W) x[(size_t)r * W + c] += v[c];
+}
+
+extern "C" int fl_add_rowvec(float* x, const float* v, int n, int W, hipStream_t stream) {
+    FL_CHECK(n >= 0 && W > 0, "add_rowvec: bad sizes");
+    if (n == 0) return 0;
+    FL_CHECK(n <= 65535, "add_rowvec: %d rows are more than one grid takes", n);
+    dim3 grid(ceil_div(W, 256), n);
+    add_rowvec_kernel<<<grid, 256, 0, stream>>>(x, v, W);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_add_rowvec)

@@ -285,3 +285,193 @@ def sample(logits, inv_temp, uniform, out):
          _check(uniform, "sample.uniform", torch.float32, (R,)),
          _check(out, "sample.out", torch.int32, (R,)), R, V, stream_handle())
     return out
+
+
+# ---------------------------------------------------------------- latent rows, recurrences, routed experts
+@dataclass
+class LatentLayerCache:
+    """The pool of one layer that keeps one row per token: ``pool[n_pages, page_size, width]``."""
+    pool: torch.Tensor
+
+    @property
+    def n_pages(self): return self.pool.shape[0]
+    @property
+    def page_size(self): return self.pool.shape[1]
+    @property
+    def width(self): return self.pool.shape[2]
+
+
+def norm_slice(x, col0, width, weight, eps, out):
+    """``out[n, width] = rmsnorm(x[:, col0 : col0 + width]) * weight`` for float32 rows ``x``."""
+    n, ld = x.shape
+    call("fl_norm_slice", _check(x, "norm_slice.x", torch.float32), ld, int(col0), int(width),
+         _check(weight, "norm_slice.weight", torch.float32, (width,)) if weight is not None else None, float(eps),
+         _check(out, "norm_slice.out", None, (n, width)), dtype_code(out.dtype), n, None, None, None, 0, 0, 0, stream_handle())
+    return out
+
+
+def norm_slice_to_pages(x, col0, width, weight, eps, cache: LatentLayerCache, positions, tok_seq, block_table):
+    """The same norm, stored into the page row of each token's position."""
+    n, ld = x.shape
+    if cache.width != width:
+        raise KernelError(f"norm_slice: rows of {width} values into a pool of rows {cache.width} wide")
+    call("fl_norm_slice", _check(x, "norm_slice.x", torch.float32), ld, int(col0), int(width),
+         _check(weight, "norm_slice.weight", torch.float32, (width,)) if weight is not None else None, float(eps),
+         _check(cache.pool, "norm_slice.pool"), dtype_code(cache.pool.dtype), n,
+         _check(positions, "norm_slice.positions", torch.int32, (n,)), _check(tok_seq, "norm_slice.tok_seq", torch.int32, (n,)),
+         _check(block_table, "norm_slice.block_table", torch.int32, (None, None)), block_table.shape[1],
+         cache.page_size, cache.n_pages, stream_handle())
+
+
+def heads_matmul(x, w, out, n_heads, transposed, gate=None, gate_col0=0):
+    """One small product per head.  ``x`` float32 ``[n, H * K]``; ``w`` ``[H * K, J]`` (``transposed`` false:
+    ``out[t, h] = x[t, h] @ w_h``) or ``[H * J, K]`` (true: ``x[t, h] @ w_h.T``); ``out`` ``[n, H * J]``.
+    ``gate``: float32 rows whose columns ``gate_col0 + h`` hold a logit per head; the head's output is
+    multiplied by its sigmoid."""
+    n, HK = x.shape
+    H = int(n_heads)
+    K = HK // H
+    J = out.shape[1] // H
+    want = (H * J, K) if transposed else (H * K, J)
+    call("fl_heads_matmul", _check(x, "heads_matmul.x", torch.float32, (n, H * K)), HK,
+         _check(w, "heads_matmul.w", None, want), dtype_code(w.dtype),
+         _check(out, "heads_matmul.out", None, (n, H * J)), dtype_code(out.dtype), n, H, K, J, int(bool(transposed)),
+         _check(gate, "heads_matmul.gate", torch.float32, (n, None)) if gate is not None else None,
+         gate.shape[1] if gate is not None else 0, int(gate_col0), stream_handle())
+    return out
+
+
+def latent_max_width() -> int:
+    from .library import load
+    return load().fl_latent_max_width()
+
+
+def latent_attention(qa, z, cache: LatentLayerCache, positions, tok_seq, block_table, n_heads, scale, window=0):
+    """``z[t, h] = sum_j softmax_j(scale * qa[t, h] . c_j) c_j`` over the cached rows of the token's request."""
+    n = qa.shape[0]
+    R = cache.width
+    call("fl_latent_attention", _check(qa, "latent_attention.qa", torch.float32, (n, n_heads * R)),
+         _check(z, "latent_attention.z", torch.float32, (n, n_heads * R)), _check(cache.pool, "latent_attention.pool"),
+         dtype_code(cache.pool.dtype), _check(positions, "latent_attention.positions", torch.int32, (n,)),
+         _check(tok_seq, "latent_attention.tok_seq", torch.int32, (n,)),
+         _check(block_table, "latent_attention.block_table", torch.int32, (None, None)), block_table.shape[1],
+         n, int(n_heads), R, cache.page_size, cache.n_pages, float(scale), int(window), stream_handle())
+    return z
+
+
+def mlstm_max_dim() -> int:
+    from .library import load
+    return load().fl_mlstm_max_dim()
+
+
+def mlstm_state_floats(dim: int, vdim: int) -> int:
+    from .library import load
+    import ctypes
+    lib = load()
+    lib.fl_mlstm_state_floats.restype = ctypes.c_long
+    lib.fl_mlstm_state_floats.argtypes = [ctypes.c_int, ctypes.c_int]
+    return int(lib.fl_mlstm_state_floats(int(dim), int(vdim)))
+
+
+def mlstm_scan(proj, cols, bias_i, bias_f, cap, q_scale, state, seq_q_start, seq_q_len, seq_slots, out, n_heads, dim, vdim):
+    """The recurrence over the step's tokens, request by request, from and into ``state``
+    ``[slots, heads, mlstm_state_floats]``.  ``proj``: float32 rows with q, k, v and the two gates'
+    pre-activations at the columns ``cols = (q, k, v, i, f)``; ``out`` float32 ``[n, heads * vdim]``."""
+    n, ld = proj.shape
+    S = seq_q_start.shape[0]
+    rec = mlstm_state_floats(dim, vdim)
+    if state.dim() != 3 or state.shape[1] != n_heads or state.shape[2] != rec:
+        raise KernelError(f"mlstm_scan.state: shape {tuple(state.shape)}, expected [slots, {n_heads}, {rec}]")
+    call("fl_mlstm_scan", _check(proj, "mlstm_scan.proj", torch.float32), ld, *(int(c) for c in cols),
+         _check(bias_i, "mlstm_scan.bias_i", torch.float32, (n_heads,)) if bias_i is not None else None,
+         _check(bias_f, "mlstm_scan.bias_f", torch.float32, (n_heads,)) if bias_f is not None else None,
+         float(cap), float(q_scale), _check(state, "mlstm_scan.state", torch.float32),
+         _check(seq_q_start, "mlstm_scan.seq_q_start", torch.int32, (S,)), _check(seq_q_len, "mlstm_scan.seq_q_len", torch.int32, (S,)),
+         _check(seq_slots, "mlstm_scan.seq_slots", torch.int32, (S,)),
+         _check(out, "mlstm_scan.out", torch.float32, (n, n_heads * vdim)), S, int(n_heads), int(dim), int(vdim), stream_handle())
+    return out
+
+
+def headnorm_gate(x, weight, gate, gate_col0, out, n_heads, eps):
+    """Every head's slice of ``x`` (float32 ``[n, H * Dv]``) divided by its root mean square, times ``weight``
+    ``[H * Dv]``, times the sigmoid of ``gate[:, gate_col0 : gate_col0 + H * Dv]``."""
+    n, HD = x.shape
+    Dv = HD // n_heads
+    call("fl_headnorm_gate", _check(x, "headnorm_gate.x", torch.float32),
+         _check(weight, "headnorm_gate.weight", torch.float32, (HD,)) if weight is not None else None,
+         _check(gate, "headnorm_gate.gate", torch.float32, (n, None)) if gate is not None else None,
+         gate.shape[1] if gate is not None else 0, int(gate_col0), _check(out, "headnorm_gate.out", None, (n, HD)),
+         dtype_code(out.dtype), n, int(n_heads), Dv, float(eps), stream_handle())
+    return out
+
+
+ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2}
+
+
+def activation(x, out, kind: str):
+    """``out = act(x)`` for float32 ``x``: ``gelu`` (with the error function), ``gelu_tanh``, ``silu``."""
+    if x.shape != out.shape:
+        raise KernelError(f"activation: shapes {tuple(x.shape)} and {tuple(out.shape)} differ")
+    call("fl_activation", _check(x, "activation.x", torch.float32), _check(out, "activation.out"), dtype_code(out.dtype),
+         x.numel(), ACTIVATIONS[kind], stream_handle())
+    return out
+
+
+def moe_tile_rows() -> int:
+    from .library import load
+    return load().fl_moe_tile_rows()
+
+
+def moe_max_tiles(n_pairs: int, n_experts: int) -> int:
+    """Upper bound of the row tiles of ``n_pairs`` (token, expert) pairs spread over ``n_experts``."""
+    return n_pairs // moe_tile_rows() + min(n_pairs, n_experts)
+
+
+def moe_route(logits, col0, n_experts, top, place, src_row, src_scale, pair_w, tiles, scoring="sigmoid", renormalise=False):
+    n, ld = logits.shape
+    P_ = n * top
+    call("fl_moe_route", _check(logits, "moe_route.logits", torch.float32), ld, int(col0), n, int(n_experts), int(top),
+         {"sigmoid": 0, "softmax": 1}[scoring], int(bool(renormalise)),
+         _check(place, "moe_route.place", torch.int32, (P_,)), _check(src_row, "moe_route.src_row", torch.int32, (P_,)),
+         _check(src_scale, "moe_route.src_scale", torch.float32, (P_,)), _check(pair_w, "moe_route.pair_w", torch.float32, (P_,)),
+         _check(tiles, "moe_route.tiles", torch.int32, (None, 4)), tiles.shape[0], stream_handle())
+
+
+def moe_gemm(x, w, out, tiles, src_row=None, src_scale=None):
+    """``out[p] = (src_scale[p] * x[src_row[p]]) @ w[e].T`` for the sorted places ``p`` of every tile, ``e`` the
+    tile's expert; ``w`` ``[E, N, K]``; without ``src_row`` the rows of ``x`` are the places themselves."""
+    E, N, K = w.shape
+    P_ = out.shape[0]
+    call("fl_moe_gemm", _check(x, "moe_gemm.x", w.dtype, (None, K)), dtype_code(w.dtype),
+         _check(src_row, "moe_gemm.src_row", torch.int32, (P_,)) if src_row is not None else None,
+         _check(src_scale, "moe_gemm.src_scale", torch.float32, (P_,)) if src_scale is not None else None,
+         _check(w, "moe_gemm.w"), _check(out, "moe_gemm.out", torch.float32, (P_, N)),
+         _check(tiles, "moe_gemm.tiles", torch.int32, (None, 4)), tiles.shape[0], N, K, stream_handle())
+    return out
+
+
+def moe_combine(y, place, top, delta, shared=None, gate=None, gate_col=0):
+    n, W = delta.shape
+    call("fl_moe_combine", _check(y, "moe_combine.y", torch.float32, (n * top, W)),
+         _check(place, "moe_combine.place", torch.int32, (n * top,)), int(top),
+         _check(shared, "moe_combine.shared", torch.float32, (n, W)) if shared is not None else None,
+         _check(gate, "moe_combine.gate", torch.float32, (n, None)) if gate is not None else None,
+         gate.shape[1] if gate is not None else 0, int(gate_col),
+         _check(delta, "moe_combine.delta", torch.float32), n, W, stream_handle())
+    return delta
+
+
+def concat_cast(a, b, out):
+    """``out = [a ; b]`` (two float32 ``[n, W]`` side by side) in ``out``'s dtype."""
+    n, W = a.shape
+    call("fl_concat_cast", _check(a, "concat.a", torch.float32), _check(b, "concat.b", torch.float32, (n, W)),
+         _check(out, "concat.out", None, (n, 2 * W)), dtype_code(out.dtype), n, W, stream_handle())
+    return out
+
+
+def add_rowvec(x, v):
+    """``x[r] += v`` for every row of the float32 ``x``."""
+    n, W = x.shape
+    call("fl_add_rowvec", _check(x, "add_rowvec.x", torch.float32), _check(v, "add_rowvec.v", torch.float32, (W,)), n, W,
+         stream_handle())
+    return x

@@ -48,6 +48,7 @@ class ModelSpec:
     head: PartSpec | None = None       # None: the plain matrix product ("linear_head"), tied or not
     eos_token_ids: tuple = ()         # every id that ends a sequence (eos_token_id is the first)
     ignored_tensors: tuple = ()       # name patterns (fnmatch) of tensors a file may hold and the model does not read
+    keeps_embedding: bool = False     # a copy of the embedding's output stays in StepState.scratch["embedding_output"] for blocks that read it
 
 
 SMALL_STEP = 16      # up to this many rows the output head runs on every row of a step
@@ -64,6 +65,11 @@ class DecoderModel:
         self.head = HEADS.create(spec.head or PartSpec("linear_head", dict(sizes, tied=spec.tied_head)))
         self._signature_mixers = None
         self._recorded_blocks = None        # per block: can its launches be recorded?
+        seen: dict = {}
+        self._visits = []                   # per run-order entry: how many earlier entries ran the same layer
+        for e in spec.run_order:
+            self._visits.append(seen.get(e.layer, 0))
+            seen[e.layer] = self._visits[-1] + 1
         for i, e in enumerate(spec.run_order):
             if not 0 <= e.layer < len(self.blocks):
                 raise ValueError(f"run-order entry {i} names layer {e.layer}, the model has {len(self.blocks)}")
@@ -178,11 +184,15 @@ class DecoderModel:
         step.scratch.clear()
         resid = rt.buffer("residual", step.n_tokens, self.spec.hidden_size, torch.float32)
         self.embedding.forward(step.tokens, resid)
+        if self.spec.keeps_embedding:
+            step.scratch["embedding_output"] = self.embedding.forward(
+                step.tokens, rt.buffer("embedding_output", step.n_tokens, self.spec.hidden_size, torch.float32))
         stream = ResidualStream(resid, rt)
         if self._recorded_blocks is None:
             self._recorded_blocks = [self._part_replayable(b) for b in self.blocks]
         for i, e in enumerate(self.spec.run_order):
             block = self.blocks[e.layer]
+            step.visit = self._visits[i]
             if step.recorder is not None and not self._recorded_blocks[e.layer]:
                 # A block that cannot be replayed ends the recorded stretch: when the step is replayed it
                 # runs again with that step's metadata.  Whatever it allocates lies elsewhere then, so

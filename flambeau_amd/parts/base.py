@@ -108,6 +108,28 @@ class PagedKVSpec(CacheSpec):
 
 
 @dataclass(frozen=True)
+class PagedRowSpec(CacheSpec):
+    """One row of ``width`` values per token, in pages: what a mixer keeps whose keys and values are
+    both made from one latent per token.  The pool of a group is ``[entries, n_pages, page_size, width]``
+    in the compute dtype.  ``window`` = number of newest rows still needed (0: all)."""
+    width: int
+    window: int = 0
+
+    def page_group(self):
+        return PageGroup(0, self.width, self.window)
+
+    def allocate_pool(self, n_entries, n_pages, page_size, dtype, device):
+        return torch.zeros((n_entries, n_pages, page_size, self.width), dtype=dtype, device=device)
+
+    def layer_view(self, pool, index):
+        from ..kernels.ops import LatentLayerCache
+        return LatentLayerCache(pool[index])
+
+    def bytes_per_token(self, element_size):
+        return self.width * element_size
+
+
+@dataclass(frozen=True)
 class StateSpec(CacheSpec):
     """Per-request state of fixed size, one record per slot, zeroed when a slot is claimed."""
     shape: tuple
@@ -145,6 +167,7 @@ class StepState:
     extra: dict = field(default_factory=dict)   # metadata parts asked for (step_metadata)
     scratch: dict = field(default_factory=dict)  # what parts compute once per forward pass and share between layers; emptied when a pass begins
     recorder: object = None        # set while the step is being recorded (engine/step.py): ``cut(fn)`` ends a recorded stretch
+    visit: int = 0                 # while a block runs: how many earlier run-order entries ran the same layer (0: its first run)
 
 
 @dataclass

@@ -8,7 +8,7 @@ which adds it, stores the sum and norms it in one kernel
 from __future__ import annotations
 
 from ..kernels import ops
-from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, PartSpec, Product
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, PartSpec, Product, TensorSpec
 
 
 class ResidualStream:
@@ -85,3 +85,81 @@ class PreNormBlock(Block):
     def forward(self, stream, step, cache):
         stream.push(self.mixer.forward(stream.normed(self.mixer_norm, lazy=self.mixer.lazy_input), step, cache))
         stream.push(self.ffn.forward(stream.normed(self.ffn_norm, lazy=self.ffn.lazy_input), step))
+
+
+@BLOCKS.register("parallel")
+class ParallelBlock(Block):
+    """One norm whose output both sublayers read: with h = Norm(x), x += Mixer(h) + FeedForward(h).
+    ``feed_forward`` may be ``None`` (a layer of a mixer alone)."""
+    replayable = True
+
+    def __init__(self, mixer: PartSpec, feed_forward: PartSpec | None, norm: PartSpec):
+        self.norm = NORMS.create(norm)
+        self.mixer = MIXERS.create(mixer)
+        self.ffn = FEED_FORWARDS.create(feed_forward) if feed_forward is not None else None
+        self._parts = {"norm": self.norm, "mixer": self.mixer}
+        if self.ffn is not None:
+            self._parts["ffn"] = self.ffn
+
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def mixers(self):
+        return [self.mixer]
+
+    def subparts(self):
+        return list(self._parts.values())
+
+    def tensors(self):
+        return {f"{p}.{name}": spec for p, part in self._parts.items() for name, spec in part.tensors().items()}
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        for p, part in self._parts.items():
+            part.bind({k[len(p) + 1:]: v for k, v in weights.items() if k.startswith(p + ".")}, rt)
+
+    def forward(self, stream, step, cache):
+        # both read the same rows, so the norm's output is a tensor (never a norm left in factors); the
+        # two deltas are added to the 32-bit stream one after the other
+        h = stream.normed(self.norm)
+        stream.push(self.mixer.forward(h, step, cache))
+        if self.ffn is not None:
+            stream.push(self.ffn.forward(h, step))
+
+
+@BLOCKS.register("stream_reentry")
+class StreamReentry(Block):
+    """What stands before a stretch of layers that runs several times: x <- W [x ; x0] + b_t, x0 the
+    embedding's output and t the number of the pass (``StepState.visit``: the block is one layer that the
+    run order names once per pass).  The model must keep the embedding's output
+    (``ModelSpec.keeps_embedding``).  No cache, no mixer."""
+    replayable = True
+
+    def __init__(self, hidden_size: int, times: int):
+        self.hidden_size = hidden_size
+        self.times = times
+
+    def mixers(self):
+        return []
+
+    def tensors(self):
+        W = self.hidden_size
+        return {"in.weight": TensorSpec((W, 2 * W)), "step.weight": TensorSpec((self.times, W), "vector32", init="normal")}
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.w_in = rt.prepare_weight(weights["in.weight"])
+        self.step_rows = [weights["step.weight"][t] for t in range(self.times)]
+
+    def forward(self, stream, step, cache):
+        rt, W = self.rt, self.hidden_size
+        resid = stream.flush()
+        x0 = step.scratch.get("embedding_output")
+        if x0 is None:
+            raise RuntimeError("stream_reentry: the model does not keep the embedding's output (ModelSpec.keeps_embedding)")
+        if not 0 <= step.visit < self.times:
+            raise RuntimeError(f"stream_reentry: pass {step.visit} of {self.times}")
+        both = rt.buffer("reentry_in", resid.shape[0], 2 * W)
+        ops.concat_cast(resid, x0, both)
+        rt.gemm(both, self.w_in, resid)
+        ops.add_rowvec(resid, self.step_rows[step.visit])

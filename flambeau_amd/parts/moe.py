@@ -1,0 +1,122 @@
+"""A feed-forward of routed experts, and the ungated feed-forward with an activation of choice.
+
+Routed: router logits z = W_r h in 32-bit, scores s = sigmoid(z) (or a softmax), the ``top`` largest
+are chosen, their scores are the weights (divided by their sum only if ``renormalise``).  An expert
+is gated, W_down (silu(W_gate u) * (W_up u)), and its weight multiplies its INPUT, u = w h
+(``weight_on="input"``), or its output.  A shared expert of the same form may run for every token and
+is added, multiplied by sigmoid(w_sg . h), one number per token.
+
+The choice never leaves the device: a kernel sorts the (token, expert) pairs by expert and cuts them
+into row tiles, the two products of all experts run as one launch each over those tiles, and a last
+kernel adds each token's experts in rising order of rank.  The router's product is the plain kernel
+(exact products, float sums), whatever the runtime's other products are.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import FEED_FORWARDS, FeedForward, Product, TensorSpec
+
+
+@FEED_FORWARDS.register("mlp")
+class Mlp(FeedForward):
+    """d = W_down act(W_up h); ``activation``: ``gelu`` (error function), ``gelu_tanh`` or ``silu``."""
+    replayable = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "gelu"):
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"mlp: unknown activation '{activation}'; known: {sorted(ops.ACTIVATIONS)}")
+        self.hidden_size, self.intermediate_size, self.activation = hidden_size, intermediate_size, activation
+
+    def tensors(self):
+        W, F = self.hidden_size, self.intermediate_size
+        return {"up.weight": TensorSpec((F, W)), "down.weight": TensorSpec((W, F))}
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.w_up = rt.prepare_weight(weights["up.weight"])
+        self.w_down = rt.prepare_weight(weights["down.weight"])
+
+    def forward(self, x, step):
+        rt, n, F = self.rt, x.shape[0], self.intermediate_size
+        pre = rt.buffer("mlp_pre", n, F, torch.float32)
+        rt.gemm(x, self.w_up, pre)
+        act = rt.buffer("mlp_act", n, F)
+        ops.activation(pre, act, self.activation)
+        return Product(act, self.w_down)
+
+
+@FEED_FORWARDS.register("routed_experts")
+class RoutedExperts(FeedForward):
+    replayable = True
+
+    def __init__(self, hidden_size: int, n_experts: int, top: int, expert_size: int, shared_size: int | None = None,
+                 scoring: str = "sigmoid", renormalise: bool = False, weight_on: str = "input", shared_gate: bool = True):
+        if weight_on not in ("input", "output"):
+            raise ValueError(f"routed_experts: weight_on must be 'input' or 'output', got {weight_on!r}")
+        if scoring not in ("sigmoid", "softmax"):
+            raise ValueError(f"routed_experts: scoring must be 'sigmoid' or 'softmax', got {scoring!r}")
+        self.hidden_size, self.n_experts, self.top = hidden_size, n_experts, top
+        self.expert_size, self.shared_size = expert_size, shared_size
+        self.scoring, self.renormalise, self.weight_on = scoring, bool(renormalise), weight_on
+        self.shared_gate = bool(shared_gate) and shared_size is not None
+
+    def tensors(self):
+        W, F = self.hidden_size, self.expert_size
+        t = {"router.weight": TensorSpec((self.n_experts, W))}
+        for e in range(self.n_experts):
+            t[f"e{e}.gate.weight"] = TensorSpec((F, W))
+            t[f"e{e}.up.weight"] = TensorSpec((F, W))
+            t[f"e{e}.down.weight"] = TensorSpec((W, F))
+        if self.shared_size is not None:
+            Fs = self.shared_size
+            t.update({"shared.gate.weight": TensorSpec((Fs, W)), "shared.up.weight": TensorSpec((Fs, W)),
+                      "shared.down.weight": TensorSpec((W, Fs))})
+            if self.shared_gate:
+                t["shared.sg.weight"] = TensorSpec((1, W))
+        return t
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        E = self.n_experts
+        # the router's rows and, behind them, the shared expert's gate: one plain product gives all logits
+        rows = [weights["router.weight"]] + ([weights["shared.sg.weight"]] if self.shared_gate else [])
+        self.w_logits = torch.cat(rows, dim=0).contiguous()
+        self.w_gate_up = torch.stack([torch.cat([weights[f"e{e}.gate.weight"], weights[f"e{e}.up.weight"]], dim=0) for e in range(E)]).contiguous()
+        self.w_down = torch.stack([weights[f"e{e}.down.weight"] for e in range(E)]).contiguous()
+        if self.shared_size is not None:
+            self.ws_gate_up = rt.prepare_gate_up(weights["shared.gate.weight"], weights["shared.up.weight"])
+            self.ws_down = rt.prepare_weight(weights["shared.down.weight"])
+
+    def forward(self, x, step):
+        rt, n = self.rt, x.shape[0]
+        W, E, top, F = self.hidden_size, self.n_experts, self.top, self.expert_size
+        pairs = n * top
+        most = rt.max_batch_tokens * top
+        logits = rt.buffer("moe_logits", n, self.w_logits.shape[0], torch.float32)
+        ops.gemm_plain(x, self.w_logits, logits)
+        ints = lambda name, rows, cols, cap: rt.buffer(name, rows, cols, torch.int32, max_rows=cap)
+        place = ints("moe_place", pairs, 1, most).view(-1)
+        src_row = ints("moe_src_row", pairs, 1, most).view(-1)
+        src_scale = rt.buffer("moe_src_scale", pairs, 1, torch.float32, max_rows=most).view(-1)
+        pair_w = rt.buffer("moe_pair_w", pairs, 1, torch.float32, max_rows=most).view(-1)
+        n_tiles = ops.moe_max_tiles(pairs, E)
+        tiles = ints("moe_tiles", n_tiles, 4, ops.moe_max_tiles(most, E))
+        ops.moe_route(logits, 0, E, top, place, src_row, src_scale, pair_w, tiles, self.scoring, self.renormalise)
+        on_input = self.weight_on == "input"
+        gate_up = rt.buffer("moe_gate_up", pairs, 2 * F, torch.float32, max_rows=most)
+        ops.moe_gemm(x, self.w_gate_up, gate_up, tiles, src_row, src_scale if on_input else None)
+        act = rt.buffer("moe_act", pairs, F, max_rows=most)
+        ops.silu_mul(gate_up, act)
+        y = rt.buffer("moe_y", pairs, W, torch.float32, max_rows=most)
+        ops.moe_gemm(act, self.w_down, y, tiles, None, None if on_input else src_scale)
+        shared = None
+        if self.shared_size is not None:
+            sact = rt.buffer("moe_shared_act", n, self.shared_size)
+            rt.gemm_swiglu(x, self.ws_gate_up, sact)
+            shared = rt.buffer("moe_shared", n, W, torch.float32)
+            rt.gemm(sact, self.ws_down, shared)
+        delta = rt.buffer("moe_delta", n, W, torch.float32)
+        ops.moe_combine(y, place, top, delta, shared=shared, gate=logits if self.shared_gate else None, gate_col=E)
+        return delta

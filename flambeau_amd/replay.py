@@ -23,7 +23,7 @@ def build_parser():
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page (divides 64)")
-    ap.add_argument("--max-slots", type=int, default=64, help="most requests live at a time")
+    ap.add_argument("--max-slots", type=int, default=4, help="most requests live at a time (state slots)")
     ap.add_argument("--plain-kernels", action="store_true",
                     help="run the plain kernels in bfloat16 too (float32 always does)")
     ap.add_argument("--poison-cache", action="store_true",
@@ -48,7 +48,7 @@ def main(argv=None) -> int:
     model, _ = load_model(args.model, dtype=args.dtype, max_batch_tokens=max_tokens,
                           tuned=not args.plain_kernels)
     runner = ModelRunner(model, n_pages=max_tokens // args.page_size, page_size=args.page_size,
-                         max_slots=args.max_slots, max_logit_rows=max_tokens)
+                         max_slots=args.max_slots, max_seq_len=max_tokens, max_logit_rows=max_tokens)
     if args.poison_cache:
         runner.storage.fill(float("nan"))
 
