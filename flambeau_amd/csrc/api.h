@@ -75,6 +75,15 @@ int fl_latent_attention(const float* qa, float* z, const void* pool, int dtype, 
                         const int* tok_seq, const int* block_table, int max_blocks, int n, int H, int R,
                         int page_size, int n_pages, float scale, int window, hipStream_t stream);
 int fl_latent_max_width(void);
+// the same on the matrix cores for bfloat16 pools (latent_tuned.hip): qa bfloat16 [n][H][R], z float [n][H][R]
+int fl_latent_attention_mfma(const void* qa, float* z, const void* pool, const int* positions,
+                             const int* tok_seq, const int* block_table, int max_blocks, int n, int H, int R,
+                             int page_size, int n_pages, float scale, int window, hipStream_t stream);
+int fl_latent_attention_mfma_takes(int R, int page_size);
+// out[t][h][j] = sum_k x[t][h][k] w[h][j][k] on the matrix cores (w bfloat16 [H][J][K])
+int fl_heads_matmul_mfma(const void* x, int x_dtype, int ldx, const void* w, void* out, int out_dtype, int n,
+                         int H, int K, int J, const float* gate, int ldg, int gate_col0, hipStream_t stream);
+int fl_heads_matmul_mfma_takes(int K, int J);
 
 // ---- the mLSTM recurrence (mlstm.hip) ----
 int fl_mlstm_scan(const float* proj, int ld, int col_q, int col_k, int col_v, int col_i, int col_f,

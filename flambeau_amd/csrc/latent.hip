@@ -14,8 +14,10 @@
 
 // ------------------------------------------------------------------ norm of a slice of columns
 // out[r, :] = v * w * rsqrt(mean(v^2) + eps), v = x[r, col0 : col0 + width] of float rows ld wide.
-// With a block table the result goes to the row of a page pool [n_pages][page_size][width] that
-// belongs to the token's position, else to the dense out[n][width].
+// With a block table the result goes to the page of the token's position, else to the dense
+// out[n][width].  A page holds its rows twice, [n_pages][2][page_size * width]: row by row
+// ([page_size][width]) and transposed ([width][page_size]); the matrix cores want the index that is
+// summed over contiguous, the latent's dims for the scores and the keys for the weighted sum.
 template <typename T>
 __global__ __launch_bounds__(256) void norm_slice_kernel(const float* __restrict__ x, int ld, int col0, int width,
                                                          const float* __restrict__ w, float eps, T* __restrict__ out,
@@ -29,15 +31,21 @@ __global__ __launch_bounds__(256) void norm_slice_kernel(const float* __restrict
     for (int i = threadIdx.x; i < width; i += 256) ss += xr[i] * xr[i];
     const float total = block_sum<4>(ss, red);
     const float inv = 1.0f / sqrtf(total / (float)width + eps);
-    T* dst;
     if (block_table) {
         const int pos = positions[r];
         const int page = block_table[(size_t)tok_seq[r] * max_blocks + pos / page_size];
         if (page < 0 || page >= n_pages) return;          // rows that pad a batch of fixed shape
-        dst = out + ((size_t)page * page_size + pos % page_size) * width;
-    } else {
-        dst = out + (size_t)r * width;
+        const int row = pos % page_size;
+        T* rows = out + (size_t)page * 2 * page_size * width;
+        T* cols = rows + (size_t)page_size * width;
+        for (int i = threadIdx.x; i < width; i += 256) {
+            const T v = from_f32<T>(xr[i] * (w ? w[i] : 1.0f) * inv);
+            rows[(size_t)row * width + i] = v;
+            cols[(size_t)i * page_size + row] = v;
+        }
+        return;
     }
+    T* dst = out + (size_t)r * width;
     for (int i = threadIdx.x; i < width; i += 256) dst[i] = from_f32<T>(xr[i] * (w ? w[i] : 1.0f) * inv);
 }
 
@@ -164,7 +172,7 @@ __global__ __launch_bounds__(64 * LA_WAVES) void latent_attention_kernel(
             float s = -INFINITY;
             if (t <= p) {
                 const int page = table[t / page_size];
-                const T* row = pool + ((size_t)page * page_size + t % page_size) * R;
+                const T* row = pool + ((size_t)page * 2 * page_size + t % page_size) * R;
                 float a = 0.f;
                 if (page >= 0 && page < n_pages)
                     for (int d = 0; d < R; ++d) a = fmaf(qh[d], to_f32(row[d]), a);
@@ -183,7 +191,7 @@ __global__ __launch_bounds__(64 * LA_WAVES) void latent_attention_kernel(
             for (int j = 0; j < cnt; ++j) {
                 const int tj = t0 + j;
                 const int page = table[tj / page_size];
-                const T* row = pool + ((size_t)page * page_size + tj % page_size) * R;
+                const T* row = pool + ((size_t)page * 2 * page_size + tj % page_size) * R;
                 const float w = ps[j];
 #pragma unroll
                 for (int u = 0; u < VPL; ++u) {

@@ -1,0 +1,252 @@
+// Attention over cached latent rows on the matrix cores (bfloat16 pools), and the small products per
+// head around it.
+//
+// A wave takes one token and up to 16 of its heads; every head of a token sees the same rows, so a
+// loaded row serves all 16.  Everything is computed transposed, as in the other attention kernels of
+// this library: S^T[key][head] = C[key][:] . Qa[head][:] (A = rows of the page, B = the folded queries,
+// held in registers for the whole walk) and Z^T[dim][head] += C^T[dim][key] P^T[key][head] (A = the
+// page's transposed copy, B = the weights, which are the lanes' own score accumulators: the rows of
+// the score tiles are dealt out so that a lane's eight values of two tiles are eight keys in a row).
+// A head is a lane column, so maxima, sums and rescaling need no broadcast.  Waves share nothing:
+// rows of different requests may lie in one block.  Keys beyond the query's position are given weight
+// zero and their values are set to zero before they are multiplied, so what an unused or reused page
+// holds (a NaN too) never reaches a sum.
+#include "common.h"
+#include "api.h"
+#include "recordable.h"
+
+#define LT_WAVES 4
+#define LT_CHUNK 64
+
+__device__ __forceinline__ bf16x8 zero_keys_beyond(bf16x8 v, int first_key, int last_visible) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+        if (first_key + e > last_visible) v[e] = (bf16_t)0.f;
+    return v;
+}
+
+// qa: bfloat16 [n][H][R]; z: float [n][H][R]; pool: [n_pages][2][page_size * R]; R = 32 * ns, ns <= NS.
+template <int NS>
+__global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_mfma_kernel(
+    const bf16_t* __restrict__ qa, float* __restrict__ z, const bf16_t* __restrict__ pool,
+    const int* __restrict__ positions, const int* __restrict__ tok_seq, const int* __restrict__ block_table,
+    int max_blocks, int n, int H, int R, int page_size, int n_pages, float scale, int window, int groups_per_token) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int unit = blockIdx.x * LT_WAVES + wave;                 // (token, group of 16 heads)
+    if (unit >= n * groups_per_token) return;
+    const int token = unit / groups_per_token, h0 = (unit - token * groups_per_token) * 16;
+    const int col = lane & 15, g = lane >> 4;                      // col: head (B columns) or row of an A tile
+    const int ns = R >> 5;
+    const int p = positions[token];
+    const int* table = block_table + (size_t)tok_seq[token] * max_blocks;
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const size_t page_stride = (size_t)2 * page_size * R;
+    const bool head_live = h0 + col < H;
+
+    // the folded queries of this lane's head, scaled: B operand of every score product
+    bf16x8 qreg[NS];
+    {
+        const bf16_t* qr = qa + ((size_t)token * H + h0 + (head_live ? col : 0)) * R;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            if (s < ns && head_live) {
+                const bf16x8 v = *(const bf16x8*)(qr + 32 * s + 8 * g);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qreg[s][e] = (bf16_t)((float)v[e] * scale);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qreg[s][e] = (bf16_t)0.f;
+            }
+        }
+    }
+    f32x4 o[2 * NS];                                               // Z^T tiles: dims 16 t + 4 g + r of head `col`
+#pragma unroll
+    for (int t = 0; t < 2 * NS; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    const int first = lo & ~(LT_CHUNK - 1);                        // chunks are aligned, so a tile of 16 keys lies in one page
+    for (int t0 = first; t0 <= p; t0 += LT_CHUNK) {
+        // ---- scores of 64 keys: four tiles of 16; tile 2 q + b, row i <-> key t0 + 32 q + 8 (i / 4) + 4 b + i % 4
+        f32x4 sacc[4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            sacc[a] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            const int key = t0 + 32 * (a >> 1) + 8 * (col >> 2) + 4 * (a & 1) + (col & 3);
+            const int kc = min(key, p);                            // a key beyond p: any loadable row, masked below
+            int page = table[kc / page_size];
+            page = min(max(page, 0), n_pages - 1);
+            const bf16_t* row = pool + (size_t)page * page_stride + (size_t)(kc % page_size) * R + 8 * g;
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+                if (s < ns) sacc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(row + 32 * s), qreg[s], sacc[a], 0, 0, 0);
+        }
+        // lane (head col, g): sacc[2 q + b][e] is key t0 + 32 q + 8 g + 4 b + e
+        float cmax = -INFINITY;
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int key = t0 + 32 * (a >> 1) + 8 * g + 4 * (a & 1) + e;
+                if (key > p || key < lo) sacc[a][e] = -INFINITY;
+                cmax = fmaxf(cmax, sacc[a][e]);
+            }
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 16, FL_WAVE));
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 32, FL_WAVE));
+        const float m_new = fmaxf(m, cmax);                        // finite: every chunk holds a visible key
+        const float corr = expf(m - m_new);
+        m = m_new;
+        bf16x8 pb[2];
+        float lsum = 0.f;
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const bf16_t w = (bf16_t)expf(sacc[a][e] - m_new);
+                pb[a >> 1][4 * (a & 1) + e] = w;
+                lsum += (float)w;                                  // the sum of the weights as they are multiplied
+            }
+        lsum += __shfl_xor(lsum, 16, FL_WAVE);
+        lsum += __shfl_xor(lsum, 32, FL_WAVE);
+        l = l * corr + lsum;
+        // ---- weighted sum: Z^T[dim][head] += C^T[dim][keys] P^T[keys][head], 32 keys a step
+        const bool edge = t0 + LT_CHUNK - 1 > p || t0 < lo;
+        const bf16_t* cols[2];
+        int key0[2];
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            key0[q] = t0 + 32 * q + 8 * g;
+            const int kc = min(key0[q], p);
+            int page = table[kc / page_size];
+            page = min(max(page, 0), n_pages - 1);
+            cols[q] = pool + (size_t)page * page_stride + (size_t)page_size * R + (key0[q] % page_size);
+        }
+#pragma unroll
+        for (int t = 0; t < 2 * NS; ++t) {
+            if (t < 2 * ns) {
+                o[t] *= corr;
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    bf16x8 v = *(const bf16x8*)(cols[q] + (size_t)(16 * t + col) * page_size);
+                    if (edge) {
+                        v = zero_keys_beyond(v, key0[q], p);
+                        if (key0[q] < lo) {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e)
+                                if (key0[q] + e < lo) v[e] = (bf16_t)0.f;
+                        }
+                    }
+                    o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pb[q], o[t], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (!head_live) return;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    float* zr = z + ((size_t)token * H + h0 + col) * R;
+#pragma unroll
+    for (int t = 0; t < 2 * NS; ++t)
+        if (t < 2 * ns) *(f32x4*)(zr + 16 * t + 4 * g) = o[t] * inv;
+}
+
+// Whether the kernel takes a pool's shape: rows of a multiple of 32 values up to 512, pages of a multiple of 16 rows.
+extern "C" int fl_latent_attention_mfma_takes(int R, int page_size) {
+    return R > 0 && R % 32 == 0 && R <= 512 && page_size > 0 && page_size % 16 == 0;
+}
+
+extern "C" int fl_latent_attention_mfma(const void* qa, float* z, const void* pool, const int* positions,
+                                        const int* tok_seq, const int* block_table, int max_blocks, int n, int H, int R,
+                                        int page_size, int n_pages, float scale, int window, hipStream_t stream) {
+    FL_CHECK(n >= 0 && H > 0 && n_pages > 0 && max_blocks > 0, "latent_attention_mfma: bad sizes");
+    FL_CHECK(fl_latent_attention_mfma_takes(R, page_size), "latent_attention_mfma: rows of %d values in pages of %d are not taken", R, page_size);
+    FL_CHECK((uintptr_t)qa % 16 == 0 && (uintptr_t)pool % 16 == 0 && (uintptr_t)z % 16 == 0, "latent_attention_mfma: operands must be 16-byte aligned");
+    FL_CHECK(window >= 0, "latent_attention_mfma: negative window");
+    if (n == 0) return 0;
+    const int groups = ceil_div(H, 16);
+    const long units = (long)n * groups;
+    FL_CHECK(units < (1L << 30), "latent_attention_mfma: too many rows");
+    const int blocks = (int)((units + LT_WAVES - 1) / LT_WAVES);
+    const int ns = R / 32;
+#define FL_LT(NS)                                                                                                       \
+    latent_attention_mfma_kernel<NS><<<blocks, 64 * LT_WAVES, 0, stream>>>((const bf16_t*)qa, z, (const bf16_t*)pool,  \
+                                                                           positions, tok_seq, block_table, max_blocks, \
+                                                                           n, H, R, page_size, n_pages, scale, window, groups)
+    if (ns <= 2) FL_LT(2);
+    else if (ns <= 4) FL_LT(4);
+    else if (ns <= 8) FL_LT(8);
+    else FL_LT(16);
+#undef FL_LT
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_latent_attention_mfma)
+
+// ------------------------------------------------------------------ one product per head on the matrix cores
+// out[t][h][j] = sum_k x[t][h][k] w[h][j][k]   (x float or bfloat16 rows ldx apart, w bfloat16 [H][J][K], K a multiple
+// of 32, J of 16), optionally times sigmoid(gate[t][gate_col0 + h]).  A wave takes 16 tokens of one head: its x is
+// the B operand, held in registers for all of K; the weights are the A operand, so a lane ends with four
+// consecutive outputs of one token.
+template <typename TX, typename TOut, int NS>
+__global__ __launch_bounds__(64 * LT_WAVES) void heads_matmul_mfma_kernel(
+    const TX* __restrict__ x, int ldx, const bf16_t* __restrict__ w, TOut* __restrict__ out, int n, int H, int K, int J,
+    const float* __restrict__ gate, int ldg, int gate_col0) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int t0 = (blockIdx.x * LT_WAVES + wave) * 16, h = blockIdx.y;
+    if (t0 >= n) return;
+    const int col = lane & 15, g = lane >> 4;
+    const int ns = K >> 5;
+    const int token = t0 + col;
+    const bool live = token < n;
+    bf16x8 xreg[NS];
+    {
+        const TX* xr = x + (size_t)(live ? token : t0) * ldx + (size_t)h * K + 8 * g;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xreg[s][e] = (s < ns && live) ? (bf16_t)to_f32(xr[32 * s + e]) : (bf16_t)0.f;
+    }
+    const float gv = (gate && live) ? 1.0f / (1.0f + expf(-gate[(size_t)token * ldg + gate_col0 + h])) : 1.0f;
+    const bf16_t* wh = w + (size_t)h * J * K;
+    for (int jt = 0; jt < J / 16; ++jt) {
+        f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+        const bf16_t* row = wh + (size_t)(16 * jt + col) * K + 8 * g;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            if (s < ns) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(row + 32 * s), xreg[s], acc, 0, 0, 0);
+        if (live) {
+            TOut* dst = out + ((size_t)token * H + h) * J + 16 * jt + 4 * g;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) dst[r] = from_f32<TOut>(acc[r] * gv);
+        }
+    }
+}
+
+extern "C" int fl_heads_matmul_mfma_takes(int K, int J) { return K > 0 && K % 32 == 0 && K <= 512 && J > 0 && J % 16 == 0; }
+
+extern "C" int fl_heads_matmul_mfma(const void* x, int x_dtype, int ldx, const void* w, void* out, int out_dtype, int n,
+                                    int H, int K, int J, const float* gate, int ldg, int gate_col0, hipStream_t stream) {
+    FL_CHECK(n >= 0 && H > 0 && ldx >= H * K, "heads_matmul_mfma: bad sizes");
+    FL_CHECK(fl_heads_matmul_mfma_takes(K, J), "heads_matmul_mfma: %d x %d per head is not taken", J, K);
+    FL_CHECK((uintptr_t)w % 16 == 0, "heads_matmul_mfma: the weights must be 16-byte aligned");
+    FL_CHECK(!gate || ldg >= gate_col0 + H, "heads_matmul_mfma: gate columns beyond rows %d wide", ldg);
+    if (n == 0) return 0;
+    FL_CHECK(H <= 65535, "heads_matmul_mfma: too many heads");
+    dim3 grid(ceil_div(n, 16 * LT_WAVES), H);
+    const int ns = K / 32;
+#define FL_HMM(TX, TO, NS) heads_matmul_mfma_kernel<TX, TO, NS><<<grid, 64 * LT_WAVES, 0, stream>>>((const TX*)x, ldx, (const bf16_t*)w, (TO*)out, n, H, K, J, gate, ldg, gate_col0)
+#define FL_HMM_NS(TX, TO)                      \
+    do {                                       \
+        if (ns <= 2) FL_HMM(TX, TO, 2);        \
+        else if (ns <= 4) FL_HMM(TX, TO, 4);   \
+        else if (ns <= 8) FL_HMM(TX, TO, 8);   \
+        else FL_HMM(TX, TO, 16);               \
+    } while (0)
+    if (x_dtype == FL_F32 && out_dtype == FL_BF16) FL_HMM_NS(float, bf16_t);
+    else if (x_dtype == FL_F32 && out_dtype == FL_F32) FL_HMM_NS(float, float);
+    else if (x_dtype == FL_BF16 && out_dtype == FL_BF16) FL_HMM_NS(bf16_t, bf16_t);
+    else FL_CHECK(false, "heads_matmul_mfma: unsupported dtypes x=%d out=%d", x_dtype, out_dtype);
+#undef FL_HMM_NS
+#undef FL_HMM
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_heads_matmul_mfma)

@@ -1,0 +1,95 @@
+"""The kernel set of attention over cached latent rows: folding the key expansion into the queries,
+attention itself, and the value expansion with the heads' gates.
+
+``PlainLatentAttention`` is the 32-bit path (and bfloat16 with the tuned kernels switched off, or at
+sizes the matrix-core kernels do not take): everything between the query projection and the output
+projection in float.  ``TunedLatentAttention`` runs each of the three on the matrix cores where its
+sizes allow (``fl_*_takes``), each on its own: the folded queries are then bfloat16, the weighted sums
+stay float."""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+from .library import call, load
+from .sets import register_kernel_set
+
+
+class LatentWeights:
+    """The expansions of one mixer as the kernels read them."""
+
+    def __init__(self, uk, uv, n_heads):
+        self.uk, self.uv, self.n_heads = uk, uv, n_heads           # [H * D, R] and [H * Dv, R], as loaded
+        self.uk_by_head = None                                      # [H, R, D]: the key expansion transposed head by head
+
+
+class PlainLatentAttention:
+    def __init__(self, rt):
+        self.rt = rt
+
+    def prepare(self, uk, uv, n_heads) -> LatentWeights:
+        return LatentWeights(uk, uv, n_heads)
+
+    def attend(self, q, w: LatentWeights, cache, step, table, scale, window, gate, gate_col0, out):
+        """``q`` float32 ``[n, H * D]`` -> ``out [n, H * Dv]`` (compute dtype): fold, attend, expand and gate."""
+        rt, n, H, R = self.rt, q.shape[0], w.n_heads, cache.width
+        qa = rt.buffer("la_qa", n, H * R, torch.float32)
+        ops.heads_matmul(q, w.uk, qa, H, transposed=False)
+        z = rt.buffer("la_z", n, H * R, torch.float32)
+        ops.latent_attention(qa, z, cache, step.positions, step.tok_seq, table, H, scale, window)
+        return ops.heads_matmul(z, w.uv, out, H, transposed=True, gate=gate, gate_col0=gate_col0)
+
+
+class TunedLatentAttention(PlainLatentAttention):
+    def prepare(self, uk, uv, n_heads):
+        w = LatentWeights(uk, uv, n_heads)
+        D, R = uk.shape[0] // n_heads, uk.shape[1]
+        if uk.dtype == torch.bfloat16 and load().fl_heads_matmul_mfma_takes(D, R):
+            w.uk_by_head = uk.view(n_heads, D, R).transpose(1, 2).contiguous()
+        return w
+
+    def attend(self, q, w, cache, step, table, scale, window, gate, gate_col0, out):
+        rt, n, H, R = self.rt, q.shape[0], w.n_heads, cache.width
+        D, Dv = q.shape[1] // H, out.shape[1] // H
+        lib = load()
+        on_cores = cache.pool.dtype == torch.bfloat16 and bool(lib.fl_latent_attention_mfma_takes(R, cache.page_size))
+        qa = rt.buffer("la_qa16" if on_cores else "la_qa", n, H * R, torch.bfloat16 if on_cores else torch.float32)
+        if w.uk_by_head is not None:
+            heads_matmul_mfma(q, w.uk_by_head, qa, H)
+        else:
+            ops.heads_matmul(q, w.uk, qa, H, transposed=False)
+        z = rt.buffer("la_z", n, H * R, torch.float32)
+        if on_cores:
+            latent_attention_mfma(qa, z, cache, step.positions, step.tok_seq, table, H, scale, window)
+        else:
+            ops.latent_attention(qa, z, cache, step.positions, step.tok_seq, table, H, scale, window)
+        if w.uv.dtype == torch.bfloat16 and lib.fl_heads_matmul_mfma_takes(R, Dv):
+            return heads_matmul_mfma(z, w.uv.view(H, Dv, R), out, H, gate=gate, gate_col0=gate_col0)
+        return ops.heads_matmul(z, w.uv, out, H, transposed=True, gate=gate, gate_col0=gate_col0)
+
+
+def heads_matmul_mfma(x, w, out, n_heads, gate=None, gate_col0=0):
+    """``out[t, h] = x[t, h] @ w[h].T`` on the matrix cores; ``w`` bfloat16 ``[H, J, K]``."""
+    n, H = x.shape[0], int(n_heads)
+    _, J, K = w.shape
+    call("fl_heads_matmul_mfma", ops._check(x, "heads_matmul.x", None, (n, H * K)), ops.dtype_code(x.dtype), H * K,
+         ops._check(w, "heads_matmul.w", torch.bfloat16, (H, J, K)), ops._check(out, "heads_matmul.out", None, (n, H * J)),
+         ops.dtype_code(out.dtype), n, H, K, J,
+         ops._check(gate, "heads_matmul.gate", torch.float32, (n, None)) if gate is not None else None,
+         gate.shape[1] if gate is not None else 0, int(gate_col0), ops.stream_handle())
+    return out
+
+
+def latent_attention_mfma(qa, z, cache, positions, tok_seq, block_table, n_heads, scale, window=0):
+    n, R = qa.shape[0], cache.width
+    call("fl_latent_attention_mfma", ops._check(qa, "latent_attention.qa", torch.bfloat16, (n, n_heads * R)),
+         ops._check(z, "latent_attention.z", torch.float32, (n, n_heads * R)),
+         ops._check(cache.pool, "latent_attention.pool", torch.bfloat16),
+         ops._check(positions, "latent_attention.positions", torch.int32, (n,)),
+         ops._check(tok_seq, "latent_attention.tok_seq", torch.int32, (n,)),
+         ops._check(block_table, "latent_attention.block_table", torch.int32, (None, None)), block_table.shape[1],
+         n, int(n_heads), R, cache.page_size, cache.n_pages, float(scale), int(window), ops.stream_handle())
+    return z
+
+
+register_kernel_set("latent_attention", PlainLatentAttention, TunedLatentAttention)

@@ -36,6 +36,8 @@ _SIGNATURES = {
     "fl_norm_slice": [P, I, I, I, P, F, P, I, I, P, P, P, I, I, I, P],
     "fl_heads_matmul": [P, I, P, I, P, I, I, I, I, I, I, P, I, I, P],
     "fl_latent_attention": [P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
+    "fl_latent_attention_mfma": [P, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
+    "fl_heads_matmul_mfma": [P, I, I, P, P, I, I, I, I, I, P, I, I, P],
     "fl_mlstm_scan": [P, I, I, I, I, I, I, P, P, F, F, P, P, P, P, P, I, I, I, I, P],
     "fl_headnorm_gate": [P, P, P, I, I, P, I, I, I, I, F, P],
     "fl_moe_route": [P, I, I, I, I, I, I, I, P, P, P, P, P, I, P],

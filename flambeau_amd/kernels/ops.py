@@ -290,15 +290,16 @@ def sample(logits, inv_temp, uniform, out):
 # ---------------------------------------------------------------- latent rows, recurrences, routed experts
 @dataclass
 class LatentLayerCache:
-    """The pool of one layer that keeps one row per token: ``pool[n_pages, page_size, width]``."""
+    """The pool of one layer that keeps one row per token: ``pool[n_pages, 2, page_size, width]``, every
+    page's rows as they are and, in its second half, transposed (``[width, page_size]``)."""
     pool: torch.Tensor
 
     @property
     def n_pages(self): return self.pool.shape[0]
     @property
-    def page_size(self): return self.pool.shape[1]
+    def page_size(self): return self.pool.shape[2]
     @property
-    def width(self): return self.pool.shape[2]
+    def width(self): return self.pool.shape[3]
 
 
 def norm_slice(x, col0, width, weight, eps, out):

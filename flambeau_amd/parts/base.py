@@ -110,8 +110,11 @@ class PagedKVSpec(CacheSpec):
 @dataclass(frozen=True)
 class PagedRowSpec(CacheSpec):
     """One row of ``width`` values per token, in pages: what a mixer keeps whose keys and values are
-    both made from one latent per token.  The pool of a group is ``[entries, n_pages, page_size, width]``
-    in the compute dtype.  ``window`` = number of newest rows still needed (0: all)."""
+    both made from one latent per token.  The pool of a group is ``[entries, n_pages, 2, page_size, width]``
+    in the compute dtype: a page holds its rows twice, row by row and (the second half, read as
+    ``[width, page_size]``) transposed, since the matrix cores want the summed-over index contiguous
+    for the scores (the dims) and for the weighted sum (the rows).  ``window`` = number of newest
+    rows still needed (0: all)."""
     width: int
     window: int = 0
 
@@ -119,14 +122,14 @@ class PagedRowSpec(CacheSpec):
         return PageGroup(0, self.width, self.window)
 
     def allocate_pool(self, n_entries, n_pages, page_size, dtype, device):
-        return torch.zeros((n_entries, n_pages, page_size, self.width), dtype=dtype, device=device)
+        return torch.zeros((n_entries, n_pages, 2, page_size, self.width), dtype=dtype, device=device)
 
     def layer_view(self, pool, index):
         from ..kernels.ops import LatentLayerCache
         return LatentLayerCache(pool[index])
 
     def bytes_per_token(self, element_size):
-        return self.width * element_size
+        return 2 * self.width * element_size
 
 
 @dataclass(frozen=True)

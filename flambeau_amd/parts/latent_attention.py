@@ -17,6 +17,7 @@ from __future__ import annotations
 import torch
 
 from ..config.base import ConfigError
+from ..kernels import latent_attention as _kernels  # noqa: F401  (registers this mixer's kernel set)
 from ..kernels import ops
 from .base import MIXERS, Mixer, PagedRowSpec, Product, TensorSpec
 
@@ -60,7 +61,8 @@ class LatentAttention(Mixer):
         self.w_low = rt.prepare_weight(torch.cat(joined, dim=0).contiguous())
         self.dq_norm, self.dkv_norm = weights["dq_norm.weight"], weights["dkv_norm.weight"]
         self.w_uq = rt.prepare_weight(weights["uq.weight"])
-        self.uk, self.uv = weights["uk.weight"], weights["uv.weight"]      # read head by head, as they are
+        self.kernels = rt.kernels("latent_attention")
+        self.expansions = self.kernels.prepare(weights["uk.weight"], weights["uv.weight"], self.n_heads)
         self.w_o = rt.prepare_weight(weights["o.weight"])
 
     def forward(self, x, step, cache):
@@ -75,10 +77,7 @@ class LatentAttention(Mixer):
             ops.norm_slice_to_pages(low, Rq, R, self.dkv_norm, self.eps, cache.kv, step.positions, step.tok_seq, table)
         q = rt.buffer("la_q", n, H * D, torch.float32)
         rt.gemm(cq, self.w_uq, q)
-        qa = rt.buffer("la_qa", n, H * R, torch.float32)
-        ops.heads_matmul(q, self.uk, qa, H, transposed=False)
-        z = rt.buffer("la_z", n, H * R, torch.float32)
-        ops.latent_attention(qa, z, cache.kv, step.positions, step.tok_seq, table, H, self.scale, self.window)
         out = rt.buffer("la_out", n, H * Dv)
-        ops.heads_matmul(z, self.uv, out, H, transposed=True, gate=low if self.gated else None, gate_col0=Rq + R)
+        self.kernels.attend(q, self.expansions, cache.kv, step, table, self.scale, self.window,
+                            low if self.gated else None, Rq + R, out)
         return Product(out, self.w_o)

@@ -60,6 +60,12 @@ CONFIGS = {
         (_att(4, 16, 16, 32, 32, 0.9), _moe(6, 4, 24, 40)),
         (_rec(4, 16, 16, 10.0), _dense(96)),
     ], loop=(0, 2, 1)), seed=21, std=0.12, page_size=16),
+    # sizes in steps of 32 and 16, which in bfloat16 run on the matrix cores: more heads than a tile of 16, pages of 16 and 32
+    "S": dict(config=_model(150, 64, 1e-5, [
+        (_att(20, 32, 16, 48, 64, 0.5), _moe(4, 2, 32, 32)),
+        (_rec(2, 32, 32, 10.0), _dense(64)),
+        (_att(4, 64, 48, 32, 96, 0.3), None),
+    ], loop=(0, 1, 2)), seed=31, std=0.15, page_size=16),
 }
 
 STORE = {"float32": torch.float32, "bfloat16": torch.bfloat16}

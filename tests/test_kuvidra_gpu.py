@@ -140,7 +140,10 @@ CUTS = ([90], [40, 5, 1, 1, 2, 20, 2, 6, 1, 12], [1] * 20 + [70])
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,D,Dv,Rq,R,scale", [(3, 8, 12, 20, 24, 0.9), (1, 40, 5, 9, 150, 0.3), (6, 4, 4, 4, 64, 2.0)])
+@pytest.mark.parametrize("H,D,Dv,Rq,R,scale", [(3, 8, 12, 20, 24, 0.9), (1, 40, 5, 9, 150, 0.3), (6, 4, 4, 4, 64, 2.0),
+                                               # sizes that the matrix-core kernels take, all three or some of them
+                                               (20, 32, 48, 24, 96, 0.7), (4, 64, 16, 40, 160, 0.04), (16, 8, 32, 8, 32, 1.0),
+                                               (2, 96, 12, 16, 512, 0.2)])
 def test_latent_attention_alone(dtype, H, D, Dv, Rq, R, scale):
     from flambeau_amd.parts import MIXERS, PartSpec
     rt = make_rt(dtype)
@@ -235,7 +238,7 @@ def test_the_stream_after_every_layer(dirs, name, dtype):
 
 # ---------------------------------------------------------------- whole models in every cutting
 LENGTHS = {"P": [40, 70, 97, 1, 33, 64, 2, 90, 55, 128, 21], "Q": [97, 1, 150, 64, 31, 2, 120, 17, 65],
-           "R": [33, 80, 5, 129, 64, 16, 100]}
+           "R": [33, 80, 5, 129, 64, 16, 100], "S": [150, 64, 3, 65, 1, 200, 31, 90]}
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
