@@ -16,6 +16,11 @@ the decode interval only, median of three repetitions.
 run in portions of 512, then 128 decoded tokens each.  ``--config 24b`` and ``--config 12b``: Mistral-Small-24B
 and Mistral-Nemo-12B sizes, 64 requests with prompts of 128 to 4,096 tokens and 256 decoded tokens each.  All go through
 ``LLMEngine`` as a serving loop would drive it and print a line of the same shape.
+
+``--config kuvidra``: the Kuvidra design (attention over cached latents, an mLSTM layer, routed experts, a looped
+stretch) at two sizes that resemble real layers, random weights, beside a Mistral of the same width, head count and
+number of layer runs: a 2,048-token prompt as one step and decode steps of 8 requests behind 2,048 tokens each.  One
+JSON line; ``value`` is Kuvidra's decode tokens/s at the larger size, the rest is under ``points``.
 """
 from __future__ import annotations
 
@@ -349,6 +354,64 @@ def bench_serving(a, name, label, cfg, dtype_name, el):
     return 0
 
 
+def kuvidra_config(width, heads, q_rank, kv_rank, ff, experts, top, expert_ff, rec_heads, rec_dim, rec_vdim, vocab=32768):
+    att = {"type": "latent_attention", "mixer": dict(heads=heads, dim=128, vdim=128, q_rank=q_rank, kv_rank=kv_rank, scale=128 ** -0.5)}
+    rec = {"type": "mlstm", "mixer": dict(heads=rec_heads, dim=rec_dim, vdim=rec_vdim, gate_cap=15.0)}
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": expert_ff}, "shared": {"ff": expert_ff}}
+    layers = [dict(att, mlp={"kind": "dense", "ff": ff}), dict(att, mlp=moe), dict(rec, mlp=moe), dict(att, mlp=moe)]
+    return {"architecture": "Kuvidra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "layers": layers,
+            "loop": {"start": 1, "stop": 3, "times": 2}}
+
+
+KUVIDRA_SIZES = {
+    "w2048": dict(width=2048, heads=16, q_rank=768, kv_rank=256, ff=8192, experts=16, top=2, expert_ff=1024,
+                  rec_heads=4, rec_dim=128, rec_vdim=256),
+    "w4096": dict(width=4096, heads=32, q_rank=1536, kv_rank=512, ff=14336, experts=32, top=4, expert_ff=1536,
+                  rec_heads=8, rec_dim=128, rec_vdim=512),
+}
+
+
+def bench_kuvidra(a, dtype_name):
+    """Prefill and decode of the Kuvidra design at layer sizes of real models, beside the closest model the engine
+    has (Mistral) at the same width, head count and number of layer runs."""
+    import torch
+    from flambeau_amd import random_model
+    points = {}
+    for name, sz in KUVIDRA_SIZES.items():
+        if a.only_size and a.only_size != name:
+            continue
+        kcfg = kuvidra_config(**sz)
+        runs = 6           # four layers, two of them twice
+        mcfg = dict(_BASE, num_hidden_layers=runs, hidden_size=sz["width"], num_attention_heads=sz["heads"], num_key_value_heads=8,
+                    head_dim=128, intermediate_size=sz["ff"], vocab_size=32768, rope_theta=1e6, sliding_window=None)
+        for label, cfg in (("kuvidra", kcfg), ("mistral", mcfg)):
+            if a.only_model and a.only_model != label:
+                continue
+            model, _ = random_model(cfg, seed=0, dtype=dtype_name, max_batch_tokens=PROMPT_LEN + 64, std=0.02, gain_std=0.0)
+            key = f"{name}_{label}"
+            if a.only in (None, "prefill"):
+                t = run_prefill(model, dtype_name)
+                points[key + "_prefill_tok_s"] = round(PROMPT_LEN / t, 1)
+                points[key + "_prefill_ms"] = round(t * 1e3, 3)
+            if a.only in (None, "decode"):
+                for b in (1, 8):
+                    dt, _ = run_decode_filled(model, b, PROMPT_LEN, steps=a.steps if a.steps < 72 else 24, warmup=min(a.warmup, 6))
+                    points[f"{key}_decode_b{b}_tok_s"] = round(b / dt, 1)
+                    points[f"{key}_decode_b{b}_ms"] = round(dt * 1e3, 3)
+            del model
+            torch.cuda.empty_cache()
+    head = points.get("w4096_kuvidra_decode_b8_tok_s")
+    out = {"metric": f"decode tok/s (Kuvidra design, width 4096, 6 layer runs, {a.dtype}, batch 8 behind 2,048 tokens)",
+           "value": head, "unit": "tokens/s", "n_gpus": 1, "steps": 24, "warmup": 6,
+           "ms_per_step": points.get("w4096_kuvidra_decode_b8_ms"), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": a.dtype, "data": "synthetic: random weights N(0, 0.02^2), uniform random token ids, caches filled with random values for decode",
+           "config": {"model": "Kuvidra design at two sizes beside Mistral of equal width", "sizes": KUVIDRA_SIZES,
+                      "global_batch": 8, "seq_len": PROMPT_LEN, "parallelism": "single GPU"},
+           "points": points}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -356,7 +419,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--reps", type=int, default=REPS, help="repetitions of the timed steps; the median is reported")
-    ap.add_argument("--config", default="7b", choices=sorted(CONFIGS))
+    ap.add_argument("--config", default="7b", choices=sorted(CONFIGS) + ["kuvidra"])
+    ap.add_argument("--only-size", default=None, choices=sorted(KUVIDRA_SIZES), help="--config kuvidra: one size only")
+    ap.add_argument("--only-model", default=None, choices=["kuvidra", "mistral"], help="--config kuvidra: one of the two models only")
     ap.add_argument("--layers", type=int, default=None, help="run only the first layers (named in config)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
@@ -371,6 +436,8 @@ def main():
     from flambeau_amd import random_model
     dtype_name = {"bf16": "bfloat16", "fp32": "float32"}[a.dtype]
     el = 2 if a.dtype == "bf16" else 4
+    if a.config == "kuvidra":
+        return bench_kuvidra(a, dtype_name)
     label, cfg = CONFIGS[a.config]
     if a.config != "7b":
         return bench_serving(a, a.config, label, cfg, dtype_name, el)

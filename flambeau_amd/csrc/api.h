@@ -78,7 +78,8 @@ int fl_latent_max_width(void);
 // the same on the matrix cores for bfloat16 pools (latent_tuned.hip): qa bfloat16 [n][H][R], z float [n][H][R]
 int fl_latent_attention_mfma(const void* qa, float* z, const void* pool, const int* positions,
                              const int* tok_seq, const int* block_table, int max_blocks, int n, int H, int R,
-                             int page_size, int n_pages, float scale, int window, hipStream_t stream);
+                             int page_size, int n_pages, float scale, int window, int n_split, float* part_o,
+                             float* part_ml, hipStream_t stream);
 int fl_latent_attention_mfma_takes(int R, int page_size);
 // out[t][h][j] = sum_k x[t][h][k] w[h][j][k] on the matrix cores (w bfloat16 [H][J][K])
 int fl_heads_matmul_mfma(const void* x, int x_dtype, int ldx, const void* w, void* out, int out_dtype, int n,
@@ -102,6 +103,12 @@ int fl_moe_route(const float* logits, int ld, int col0, int n, int E, int top, i
 int fl_moe_tile_rows(void);
 int fl_moe_gemm(const void* x, int dtype, const int* src_row, const float* src_scale, const void* w,
                 float* out, const int* tiles, int max_tiles, int N, int K, hipStream_t stream);
+// fl_moe_gemm on the matrix cores (bfloat16 x and w; moe_tuned.hip)
+int fl_moe_gemm_mfma(const void* x, const int* src_row, const float* src_scale, const void* w, float* out,
+                     const int* tiles, int max_tiles, int N, int K, hipStream_t stream);
+int fl_moe_gemm_mfma_takes(int N, int K);
+// out[m][f] = sum_k x[m][k] w[f][k] for few features f: one wave per output, float sums in a fixed order
+int fl_gemm_few(const void* x, const void* w, float* out, int dtype, int M, int N, int K, hipStream_t stream);
 int fl_moe_combine(const float* y, const int* place, int top, const float* shared, const float* gate, int ldg,
                    int gate_col, float* delta, int n, int W, hipStream_t stream);
 int fl_activation(const float* x, void* out, int out_dtype, long total, int kind, hipStream_t stream);

@@ -26,15 +26,19 @@ __device__ __forceinline__ bf16x8 zero_keys_beyond(bf16x8 v, int first_key, int 
 }
 
 // qa: bfloat16 [n][H][R]; z: float [n][H][R]; pool: [n_pages][2][page_size * R]; R = 32 * ns, ns <= NS.
+// n_split > 1: the keys of every token are dealt out to that many waves, which leave their sums in
+// part_o [n * groups * n_split * 16][R] and (maximum, sum of weights) in part_ml [...][2]; a second kernel adds them.
 template <int NS>
 __global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_mfma_kernel(
     const bf16_t* __restrict__ qa, float* __restrict__ z, const bf16_t* __restrict__ pool,
     const int* __restrict__ positions, const int* __restrict__ tok_seq, const int* __restrict__ block_table,
-    int max_blocks, int n, int H, int R, int page_size, int n_pages, float scale, int window, int groups_per_token) {
+    int max_blocks, int n, int H, int R, int page_size, int n_pages, float scale, int window, int groups_per_token,
+    int n_split, float* __restrict__ part_o, float* __restrict__ part_ml) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int unit = blockIdx.x * LT_WAVES + wave;                 // (token, group of 16 heads)
-    if (unit >= n * groups_per_token) return;
-    const int token = unit / groups_per_token, h0 = (unit - token * groups_per_token) * 16;
+    const int unit = blockIdx.x * LT_WAVES + wave;                 // (token, group of 16 heads, part of the keys)
+    if (unit >= n * groups_per_token * n_split) return;
+    const int split = unit % n_split, tg = unit / n_split;
+    const int token = tg / groups_per_token, h0 = (tg - token * groups_per_token) * 16;
     const int col = lane & 15, g = lane >> 4;                      // col: head (B columns) or row of an A tile
     const int ns = R >> 5;
     const int p = positions[token];
@@ -64,8 +68,15 @@ __global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_mfma_kernel(
     for (int t = 0; t < 2 * NS; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
-    const int first = lo & ~(LT_CHUNK - 1);                        // chunks are aligned, so a tile of 16 keys lies in one page
-    for (int t0 = first; t0 <= p; t0 += LT_CHUNK) {
+    int first = lo & ~(LT_CHUNK - 1);                              // chunks are aligned, so a tile of 16 keys lies in one page
+    int last = p;
+    if (n_split > 1) {
+        // this part's chunks: the token's chunks dealt out in equal runs (a short context leaves late parts empty)
+        const int chunks = (p - first) / LT_CHUNK + 1, per = (chunks + n_split - 1) / n_split;
+        last = min(p, first + (split + 1) * per * LT_CHUNK - 1);
+        first += split * per * LT_CHUNK;
+    }
+    for (int t0 = first; t0 <= last; t0 += LT_CHUNK) {
         // ---- scores of 64 keys: four tiles of 16; tile 2 q + b, row i <-> key t0 + 32 q + 8 (i / 4) + 4 b + i % 4
         f32x4 sacc[4];
 #pragma unroll
@@ -140,12 +151,50 @@ __global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_mfma_kernel(
             }
         }
     }
+    if (n_split > 1) {
+        // unnormalised sums relative to this part's own maximum; fl_latent_attention_mfma's second kernel adds the parts
+        float* po = part_o + ((size_t)unit * 16 + col) * R;
+#pragma unroll
+        for (int t = 0; t < 2 * NS; ++t)
+            if (t < 2 * ns) *(f32x4*)(po + 16 * t + 4 * g) = o[t];
+        if (g == 0) {
+            part_ml[((size_t)unit * 16 + col) * 2] = m;
+            part_ml[((size_t)unit * 16 + col) * 2 + 1] = l;
+        }
+        return;
+    }
     if (!head_live) return;
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     float* zr = z + ((size_t)token * H + h0 + col) * R;
 #pragma unroll
     for (int t = 0; t < 2 * NS; ++t)
         if (t < 2 * ns) *(f32x4*)(zr + 16 * t + 4 * g) = o[t] * inv;
+}
+
+// z[token][head][:] = sum_s o_s exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s, over the parts of the keys
+// (rising s; an empty part has m = -inf and adds nothing).  One wave per (token, head).
+__global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                           float* __restrict__ z, int total, int H, int R, int groups, int n_split) {
+    const int unit = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (unit >= total) return;
+    const int token = unit / H, h = unit - token * H;
+    const size_t base = ((size_t)(token * groups + (h >> 4)) * n_split) * 16 + (h & 15);        // part 0; parts are 16 rows apart
+    float M = -INFINITY;
+    for (int s = 0; s < n_split; ++s) M = fmaxf(M, part_ml[(base + (size_t)s * 16) * 2]);
+    float L = 0.f;
+    for (int s = 0; s < n_split; ++s) {
+        const float ms = part_ml[(base + (size_t)s * 16) * 2];
+        if (ms > -INFINITY) L += part_ml[(base + (size_t)s * 16) * 2 + 1] * expf(ms - M);
+    }
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    for (int d = lane; d < R; d += 64) {
+        float acc = 0.f;
+        for (int s = 0; s < n_split; ++s) {
+            const float ms = part_ml[(base + (size_t)s * 16) * 2];
+            if (ms > -INFINITY) acc += part_o[(base + (size_t)s * 16) * R + d] * expf(ms - M);
+        }
+        z[(size_t)unit * R + d] = acc * inv;
+    }
 }
 
 // Whether the kernel takes a pool's shape: rows of a multiple of 32 values up to 512, pages of a multiple of 16 rows.
@@ -155,27 +204,35 @@ extern "C" int fl_latent_attention_mfma_takes(int R, int page_size) {
 
 extern "C" int fl_latent_attention_mfma(const void* qa, float* z, const void* pool, const int* positions,
                                         const int* tok_seq, const int* block_table, int max_blocks, int n, int H, int R,
-                                        int page_size, int n_pages, float scale, int window, hipStream_t stream) {
+                                        int page_size, int n_pages, float scale, int window, int n_split, float* part_o,
+                                        float* part_ml, hipStream_t stream) {
     FL_CHECK(n >= 0 && H > 0 && n_pages > 0 && max_blocks > 0, "latent_attention_mfma: bad sizes");
+    FL_CHECK(n_split >= 1 && (n_split == 1 || (part_o && part_ml)), "latent_attention_mfma: %d parts of the keys need a workspace", n_split);
     FL_CHECK(fl_latent_attention_mfma_takes(R, page_size), "latent_attention_mfma: rows of %d values in pages of %d are not taken", R, page_size);
     FL_CHECK((uintptr_t)qa % 16 == 0 && (uintptr_t)pool % 16 == 0 && (uintptr_t)z % 16 == 0, "latent_attention_mfma: operands must be 16-byte aligned");
     FL_CHECK(window >= 0, "latent_attention_mfma: negative window");
     if (n == 0) return 0;
     const int groups = ceil_div(H, 16);
-    const long units = (long)n * groups;
+    const long units = (long)n * groups * n_split;
     FL_CHECK(units < (1L << 30), "latent_attention_mfma: too many rows");
     const int blocks = (int)((units + LT_WAVES - 1) / LT_WAVES);
     const int ns = R / 32;
 #define FL_LT(NS)                                                                                                       \
     latent_attention_mfma_kernel<NS><<<blocks, 64 * LT_WAVES, 0, stream>>>((const bf16_t*)qa, z, (const bf16_t*)pool,  \
                                                                            positions, tok_seq, block_table, max_blocks, \
-                                                                           n, H, R, page_size, n_pages, scale, window, groups)
+                                                                           n, H, R, page_size, n_pages, scale, window, groups, \
+                                                                           n_split, part_o, part_ml)
     if (ns <= 2) FL_LT(2);
     else if (ns <= 4) FL_LT(4);
     else if (ns <= 8) FL_LT(8);
     else FL_LT(16);
 #undef FL_LT
     FL_LAUNCH_CHECK();
+    if (n_split > 1) {
+        const int total = n * H;
+        latent_merge_kernel<<<(total + 3) / 4, 256, 0, stream>>>(part_o, part_ml, z, total, H, R, groups, n_split);
+        FL_LAUNCH_CHECK();
+    }
     return 0;
 }
 FL_RECORDABLE(fl_latent_attention_mfma)

@@ -14,7 +14,7 @@
 
 #define ML_GROUP 16          // threads that share a column of S; they own the rows d = g, g + 16, ...
 #define ML_COLS 16           // columns of S per block
-#define ML_MAX_ROWS 16       // rows per thread: D <= ML_GROUP * ML_MAX_ROWS
+#define ML_MAX_ROWS 32       // rows per thread: D <= ML_GROUP * ML_MAX_ROWS
 
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
@@ -22,8 +22,10 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - l
 // the gate pre-activations zi [H] at col_i, zf [H] at col_f.
 // Block = (columns j0 .. j0 + 15, head, request); thread (g, c) holds S[d][j0 + c] for its rows d.
 // Every block walks n and m for itself and keeps a copy of its own in the state, since blocks of one
-// head start and end at different times: state [slots][H][D * Dv + blocks * (D + 1)], S first, then
-// per block of columns n [D] and m (fl_mlstm_state_floats gives the record's size).
+// head start and end at different times: state [slots][H][D * Dv + blocks * (D + 1)], S first (column by
+// column, S[d][j] at j * D + d, so that the threads of a column read neighbours), then per block of
+// columns n [D] and m (fl_mlstm_state_floats gives the record's size).  A token's inputs are fetched
+// while the token before it is worked on.
 template <int RPT>
 __global__ __launch_bounds__(ML_GROUP * ML_COLS) void mlstm_scan_kernel(
     const float* __restrict__ proj, int ld, int col_q, int col_k, int col_v, int col_i, int col_f,
@@ -41,23 +43,32 @@ __global__ __launch_bounds__(ML_GROUP * ML_COLS) void mlstm_scan_kernel(
 #pragma unroll
     for (int u = 0; u < RPT; ++u) {
         const int d = g + ML_GROUP * u;
-        S[u] = (live && d < D) ? st[(size_t)d * Dv + j] : 0.f;
+        S[u] = (live && d < D) ? st[(size_t)j * D + d] : 0.f;
         nn[u] = d < D ? mine[d] : 0.f;
     }
     float m = mine[D];
     const float bi = bias_i ? bias_i[head] : 0.f, bf = bias_f ? bias_f[head] : 0.f;
-    for (int t = 0; t < len; ++t) {
+    float q[RPT], k[RPT], v = 0.f, zi = 0.f, zf = 0.f;
+    auto fetch = [&](int t, float* qn, float* kn, float& vn, float& zin, float& zfn) {
         const float* row = proj + (size_t)(start + t) * ld;
-        float q[RPT], k[RPT];
 #pragma unroll
         for (int u = 0; u < RPT; ++u) {
             const int d = g + ML_GROUP * u;
-            q[u] = d < D ? row[col_q + head * D + d] * q_scale : 0.f;
-            k[u] = d < D ? row[col_k + head * D + d] : 0.f;
+            qn[u] = d < D ? row[col_q + head * D + d] : 0.f;
+            kn[u] = d < D ? row[col_k + head * D + d] : 0.f;
         }
-        const float v = live ? row[col_v + head * Dv + j] : 0.f;
-        const float gi = cap * tanhf((row[col_i + head] + bi) / cap);
-        const float gf = log_sigmoid(cap * tanhf((row[col_f + head] + bf) / cap));
+        vn = live ? row[col_v + head * Dv + j] : 0.f;
+        zin = row[col_i + head];
+        zfn = row[col_f + head];
+    };
+    if (len > 0) fetch(0, q, k, v, zi, zf);
+    for (int t = 0; t < len; ++t) {
+        float qn[RPT], kn[RPT], vn = 0.f, zin = 0.f, zfn = 0.f;
+        if (t + 1 < len) fetch(t + 1, qn, kn, vn, zin, zfn);
+#pragma unroll
+        for (int u = 0; u < RPT; ++u) q[u] *= q_scale;
+        const float gi = cap * tanhf((zi + bi) / cap);
+        const float gf = log_sigmoid(cap * tanhf((zf + bf) / cap));
         const float m_new = fmaxf(gf + m, gi);
         const float a = expf(gf + m - m_new), b = expf(gi - m_new);
         m = m_new;
@@ -75,11 +86,16 @@ __global__ __launch_bounds__(ML_GROUP * ML_COLS) void mlstm_scan_kernel(
             den += __shfl_xor(den, off, FL_WAVE);
         }
         if (live && g == 0) out[((size_t)(start + t) * H + head) * Dv + j] = num / (fmaxf(fabsf(den), expf(-m)) + 1e-6f);
+        if (t + 1 < len) {
+#pragma unroll
+            for (int u = 0; u < RPT; ++u) { q[u] = qn[u]; k[u] = kn[u]; }
+            v = vn; zi = zin; zf = zfn;
+        }
     }
 #pragma unroll
     for (int u = 0; u < RPT; ++u) {
         const int d = g + ML_GROUP * u;
-        if (live && d < D) st[(size_t)d * Dv + j] = S[u];
+        if (live && d < D) st[(size_t)j * D + d] = S[u];
         if (c == 0 && d < D) mine[d] = nn[u];
     }
     if (threadIdx.x == 0) mine[D] = m;
@@ -110,6 +126,7 @@ extern "C" int fl_mlstm_scan(const float* proj, int ld, int col_q, int col_k, in
     else if (rpt <= 2) FL_ML(2);
     else if (rpt <= 4) FL_ML(4);
     else if (rpt <= 8) FL_ML(8);
+    else if (rpt <= 16) FL_ML(16);
     else FL_ML(ML_MAX_ROWS);
 #undef FL_ML
     FL_LAUNCH_CHECK();

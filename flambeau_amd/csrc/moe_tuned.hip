@@ -1,0 +1,147 @@
+// The experts' products on the matrix cores (bfloat16), and a product with few output features.
+#include "common.h"
+#include "api.h"
+#include "recordable.h"
+
+#define MT_TILE 64            // rows of a tile (fl_moe_route cuts the sorted pairs into tiles of this many)
+#define MT_FEATURES 128       // output features per block: four waves of 32
+
+// out[p][:] = (scale[p] * x[src[p]]) W_e^T over the tiles of fl_moe_route, as fl_moe_gemm computes it, with
+// v_mfma_f32_16x16x32_bf16: a wave takes 32 features (two A operands, read straight from the expert's
+// rows) against up to four groups of 16 rows (B operands); K in steps of 32.  Row groups a tile does not
+// have are skipped, so a decode step (a row or two per expert) streams the weights once.
+__global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __restrict__ x, const int* __restrict__ src_row,
+                                                            const float* __restrict__ src_scale, const bf16_t* __restrict__ w,
+                                                            float* __restrict__ out, const int* __restrict__ tiles, int N, int K) {
+    const int e = tiles[4 * blockIdx.y + 0];
+    if (e < 0) return;
+    const int p0 = tiles[4 * blockIdx.y + 1], M = tiles[4 * blockIdx.y + 2];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int col = lane & 15, g = lane >> 4;
+    const int f0 = blockIdx.x * MT_FEATURES + wave * 32;
+    if (f0 >= N) return;
+    const bf16_t* we = w + (size_t)e * N * K;
+    const bf16_t* wrow[2];
+    bool wlive[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+        const int f = f0 + 16 * a + col;
+        wlive[a] = f < N;
+        wrow[a] = we + (size_t)(wlive[a] ? f : 0) * K + 8 * g;
+    }
+    const int groups = (M + 15) >> 4;
+    const bf16_t* xrow[4];
+    float xs[4];
+    bool xlive[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int r = 16 * t + col;
+        xlive[t] = r < M;
+        const int p = p0 + (xlive[t] ? r : 0);
+        xrow[t] = x + (size_t)(src_row ? src_row[p] : p) * K + 8 * g;
+        xs[t] = src_scale ? src_scale[p] : 1.0f;
+    }
+    f32x4 acc[2][4];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[a][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const bf16x8 zero = {(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        bf16x8 av[2], bv[4];
+#pragma unroll
+        for (int a = 0; a < 2; ++a) av[a] = wlive[a] ? *(const bf16x8*)(wrow[a] + k0) : zero;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            if (t < groups) {
+                bv[t] = xlive[t] ? *(const bf16x8*)(xrow[t] + k0) : zero;
+                if (src_scale) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) bv[t][i] = (bf16_t)((float)bv[t][i] * xs[t]);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (t < groups) {
+#pragma unroll
+                for (int a = 0; a < 2; ++a) acc[a][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[a], bv[t], acc[a][t], 0, 0, 0);
+            }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        if (!xlive[t] || t >= groups) continue;
+        float* dst = out + (size_t)(p0 + 16 * t + col) * N;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            const int f = f0 + 16 * a + 4 * g;
+            if (f + 3 < N) {
+                *(f32x4*)(dst + f) = acc[a][t];
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (f + r < N) dst[f + r] = acc[a][t][r];
+            }
+        }
+    }
+}
+
+extern "C" int fl_moe_gemm_mfma_takes(int N, int K) { return N > 0 && N % 4 == 0 && K > 0 && K % 32 == 0; }
+
+extern "C" int fl_moe_gemm_mfma(const void* x, const int* src_row, const float* src_scale, const void* w, float* out,
+                                const int* tiles, int max_tiles, int N, int K, hipStream_t stream) {
+    FL_CHECK(max_tiles >= 0 && fl_moe_gemm_mfma_takes(N, K), "moe_gemm_mfma: %d features over %d values are not taken", N, K);
+    FL_CHECK((uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0, "moe_gemm_mfma: operands must be 16-byte aligned");
+    if (max_tiles == 0) return 0;
+    FL_CHECK(max_tiles <= 65535, "moe_gemm_mfma: %d row tiles are more than one grid takes", max_tiles);
+    dim3 grid(ceil_div(N, MT_FEATURES), max_tiles);
+    moe_gemm_mfma_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)x, src_row, src_scale, (const bf16_t*)w, out, tiles, N, K);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_moe_gemm_mfma)
+
+// ------------------------------------------------------------------ a product with few output features
+// out[m][f] = sum_k x[m][k] w[f][k] for a handful of features (a router's scores, a gate's logit): one
+// wave per output element, the lanes stride over k and add their parts in a fixed tree, so an element
+// does not depend on how many rows the call has.  Products of stored values are exact in float; the
+// sums are float.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_few_kernel(const T* __restrict__ x, const T* __restrict__ w, float* __restrict__ out,
+                                                       long total, int N, int K) {
+    const long unit = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (unit >= total) return;
+    const int lane = threadIdx.x & 63;
+    const long m = unit / N;
+    const int f = (int)(unit - m * N);
+    const T* xr = x + (size_t)m * K;
+    const T* wr = w + (size_t)f * K;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int k = 4 * lane;
+    if (K % 4 == 0) {
+        for (; k + 3 < K; k += 256) {
+            a0 = fmaf(to_f32(xr[k]), to_f32(wr[k]), a0);
+            a1 = fmaf(to_f32(xr[k + 1]), to_f32(wr[k + 1]), a1);
+            a2 = fmaf(to_f32(xr[k + 2]), to_f32(wr[k + 2]), a2);
+            a3 = fmaf(to_f32(xr[k + 3]), to_f32(wr[k + 3]), a3);
+        }
+    } else {
+        for (k = lane; k < K; k += 64) a0 = fmaf(to_f32(xr[k]), to_f32(wr[k]), a0);
+    }
+    const float s = wave_sum((a0 + a1) + (a2 + a3));
+    if (lane == 0) out[unit] = s;
+}
+
+extern "C" int fl_gemm_few(const void* x, const void* w, float* out, int dtype, int M, int N, int K, hipStream_t stream) {
+    FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_few: bad sizes M=%d N=%d K=%d", M, N, K);
+    if (M == 0) return 0;
+    const long total = (long)M * N;
+    const long blocks = (total + 3) / 4;
+    FL_CHECK(blocks < (1L << 31), "gemm_few: too many outputs");
+    if (dtype == FL_F32) gemm_few_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)x, (const float*)w, out, total, N, K);
+    else if (dtype == FL_BF16) gemm_few_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, total, N, K);
+    else FL_CHECK(false, "gemm_few: unknown dtype %d", dtype);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_gemm_few)

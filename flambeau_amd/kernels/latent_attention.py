@@ -39,8 +39,28 @@ class PlainLatentAttention:
         ops.latent_attention(qa, z, cache, step.positions, step.tok_seq, table, H, scale, window)
         return ops.heads_matmul(z, w.uv, out, H, transposed=True, gate=gate, gate_col0=gate_col0)
 
+    def signature(self, batch, n_heads: int):
+        """What the kernels decide from the contexts' lengths (part of a recorded step's key)."""
+        return ()
+
+
+SPLIT_TARGET_WAVES = 1024     # four per compute unit
+SPLIT_MIN_KEYS = 128          # a part of the keys is at least two chunks of 64
+
+
+def key_splits(batch, n_heads: int) -> int:
+    """Into how many parts the matrix-core kernel deals the keys of every token: a step of few rows
+    behind long contexts (decoding) has too few (token, 16 heads) units to fill the chip."""
+    units = batch.n_tokens * -(-n_heads // 16)
+    most = max(1, batch.max_ctx_len // SPLIT_MIN_KEYS)
+    parts = max(1, min(SPLIT_TARGET_WAVES // max(units, 1), most, 64))
+    return 1 << (parts.bit_length() - 1)          # a power of two: few different launches while contexts grow
+
 
 class TunedLatentAttention(PlainLatentAttention):
+    def signature(self, batch, n_heads):
+        return key_splits(batch, n_heads)
+
     def prepare(self, uk, uv, n_heads):
         w = LatentWeights(uk, uv, n_heads)
         D, R = uk.shape[0] // n_heads, uk.shape[1]
@@ -60,7 +80,13 @@ class TunedLatentAttention(PlainLatentAttention):
             ops.heads_matmul(q, w.uk, qa, H, transposed=False)
         z = rt.buffer("la_z", n, H * R, torch.float32)
         if on_cores:
-            latent_attention_mfma(qa, z, cache, step.positions, step.tok_seq, table, H, scale, window)
+            n_split = key_splits(step.host, H)
+            part_o = part_ml = None
+            if n_split > 1:
+                rows = n * -(-H // 16) * n_split * 16
+                part_o = rt.buffer("la_part_o", rows, R, torch.float32, max_rows=16 * (SPLIT_TARGET_WAVES + 64))
+                part_ml = rt.buffer("la_part_ml", rows, 2, torch.float32, max_rows=16 * (SPLIT_TARGET_WAVES + 64))
+            latent_attention_mfma(qa, z, cache, step.positions, step.tok_seq, table, H, scale, window, n_split, part_o, part_ml)
         else:
             ops.latent_attention(qa, z, cache, step.positions, step.tok_seq, table, H, scale, window)
         if w.uv.dtype == torch.bfloat16 and lib.fl_heads_matmul_mfma_takes(R, Dv):
@@ -80,15 +106,25 @@ def heads_matmul_mfma(x, w, out, n_heads, gate=None, gate_col0=0):
     return out
 
 
-def latent_attention_mfma(qa, z, cache, positions, tok_seq, block_table, n_heads, scale, window=0):
+def latent_attention_mfma(qa, z, cache, positions, tok_seq, block_table, n_heads, scale, window=0, n_split=1,
+                          part_o=None, part_ml=None):
+    """``n_split`` > 1: every token's keys are dealt out to that many waves; ``part_o`` (float32, at least
+    ``n * ceil(H / 16) * n_split * 16`` rows of R) and ``part_ml`` (as many rows of 2) hold their sums."""
     n, R = qa.shape[0], cache.width
+    if n_split > 1:
+        rows = n * -(-n_heads // 16) * n_split * 16
+        ops._check(part_o, "latent_attention.part_o", torch.float32, (None, R))
+        ops._check(part_ml, "latent_attention.part_ml", torch.float32, (None, 2))
+        if part_o.shape[0] < rows or part_ml.shape[0] < rows:
+            raise ops.KernelError(f"latent_attention: {n_split} parts need {rows} rows of workspace")
     call("fl_latent_attention_mfma", ops._check(qa, "latent_attention.qa", torch.bfloat16, (n, n_heads * R)),
          ops._check(z, "latent_attention.z", torch.float32, (n, n_heads * R)),
          ops._check(cache.pool, "latent_attention.pool", torch.bfloat16),
          ops._check(positions, "latent_attention.positions", torch.int32, (n,)),
          ops._check(tok_seq, "latent_attention.tok_seq", torch.int32, (n,)),
          ops._check(block_table, "latent_attention.block_table", torch.int32, (None, None)), block_table.shape[1],
-         n, int(n_heads), R, cache.page_size, cache.n_pages, float(scale), int(window), ops.stream_handle())
+         n, int(n_heads), R, cache.page_size, cache.n_pages, float(scale), int(window), int(n_split),
+         part_o.data_ptr() if n_split > 1 else None, part_ml.data_ptr() if n_split > 1 else None, ops.stream_handle())
     return z
 
 

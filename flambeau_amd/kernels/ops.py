@@ -438,11 +438,30 @@ def moe_route(logits, col0, n_experts, top, place, src_row, src_scale, pair_w, t
          _check(tiles, "moe_route.tiles", torch.int32, (None, 4)), tiles.shape[0], stream_handle())
 
 
-def moe_gemm(x, w, out, tiles, src_row=None, src_scale=None):
+def gemm_few(x, w, out):
+    """``out[m, f] = sum_k x[m, k] w[f, k]`` (float32 ``out``) for a handful of features: one wave per output."""
+    M, K = x.shape
+    N = w.shape[0]
+    call("fl_gemm_few", _check(x, "gemm_few.x", w.dtype, (M, K)), _check(w, "gemm_few.w", None, (N, K)),
+         _check(out, "gemm_few.out", torch.float32, (M, N)), dtype_code(x.dtype), M, N, K, stream_handle())
+    return out
+
+
+def moe_gemm(x, w, out, tiles, src_row=None, src_scale=None, matrix_cores=False):
     """``out[p] = (src_scale[p] * x[src_row[p]]) @ w[e].T`` for the sorted places ``p`` of every tile, ``e`` the
-    tile's expert; ``w`` ``[E, N, K]``; without ``src_row`` the rows of ``x`` are the places themselves."""
+    tile's expert; ``w`` ``[E, N, K]``; without ``src_row`` the rows of ``x`` are the places themselves.
+    ``matrix_cores``: the bfloat16 kernel on the matrix cores where it takes the sizes."""
     E, N, K = w.shape
     P_ = out.shape[0]
+    if matrix_cores and w.dtype == torch.bfloat16:
+        from .library import load
+        if load().fl_moe_gemm_mfma_takes(N, K):
+            call("fl_moe_gemm_mfma", _check(x, "moe_gemm.x", w.dtype, (None, K)),
+                 _check(src_row, "moe_gemm.src_row", torch.int32, (P_,)) if src_row is not None else None,
+                 _check(src_scale, "moe_gemm.src_scale", torch.float32, (P_,)) if src_scale is not None else None,
+                 _check(w, "moe_gemm.w"), _check(out, "moe_gemm.out", torch.float32, (P_, N)),
+                 _check(tiles, "moe_gemm.tiles", torch.int32, (None, 4)), tiles.shape[0], N, K, stream_handle())
+            return out
     call("fl_moe_gemm", _check(x, "moe_gemm.x", w.dtype, (None, K)), dtype_code(w.dtype),
          _check(src_row, "moe_gemm.src_row", torch.int32, (P_,)) if src_row is not None else None,
          _check(src_scale, "moe_gemm.src_scale", torch.float32, (P_,)) if src_scale is not None else None,

@@ -39,10 +39,11 @@ class LatentAttention(Mixer):
         return PagedRowSpec(self.kv_rank, self.window)
 
     def signature_group(self):
-        return ("latent_attention",)
+        return ("latent_attention", self.n_heads)
 
     def step_signature(self, batch):
-        return ()           # the kernels' launches follow from the batch's shape alone
+        """Into how many parts the kernels deal the keys: all that this mixer decides from the contexts' lengths."""
+        return self.kernels.signature(batch, self.n_heads)
 
     def tensors(self):
         W, H, D, Dv, Rq, R = self.hidden_size, self.n_heads, self.head_dim, self.value_dim, self.q_rank, self.kv_rank

@@ -8,8 +8,9 @@ is added, multiplied by sigmoid(w_sg . h), one number per token.
 
 The choice never leaves the device: a kernel sorts the (token, expert) pairs by expert and cuts them
 into row tiles, the two products of all experts run as one launch each over those tiles, and a last
-kernel adds each token's experts in rising order of rank.  The router's product is the plain kernel
-(exact products, float sums), whatever the runtime's other products are.
+kernel adds each token's experts in rising order of rank.  The router's product is a kernel of its own
+(one wave per score: exact products, float sums in a fixed order), whatever the runtime's other products
+are; the experts' products run on the matrix cores in bfloat16 and as plain products in 32-bit.
 """
 from __future__ import annotations
 
@@ -95,7 +96,7 @@ class RoutedExperts(FeedForward):
         pairs = n * top
         most = rt.max_batch_tokens * top
         logits = rt.buffer("moe_logits", n, self.w_logits.shape[0], torch.float32)
-        ops.gemm_plain(x, self.w_logits, logits)
+        ops.gemm_few(x, self.w_logits, logits)
         ints = lambda name, rows, cols, cap: rt.buffer(name, rows, cols, torch.int32, max_rows=cap)
         place = ints("moe_place", pairs, 1, most).view(-1)
         src_row = ints("moe_src_row", pairs, 1, most).view(-1)
@@ -106,11 +107,11 @@ class RoutedExperts(FeedForward):
         ops.moe_route(logits, 0, E, top, place, src_row, src_scale, pair_w, tiles, self.scoring, self.renormalise)
         on_input = self.weight_on == "input"
         gate_up = rt.buffer("moe_gate_up", pairs, 2 * F, torch.float32, max_rows=most)
-        ops.moe_gemm(x, self.w_gate_up, gate_up, tiles, src_row, src_scale if on_input else None)
+        ops.moe_gemm(x, self.w_gate_up, gate_up, tiles, src_row, src_scale if on_input else None, matrix_cores=rt.tuned)
         act = rt.buffer("moe_act", pairs, F, max_rows=most)
         ops.silu_mul(gate_up, act)
         y = rt.buffer("moe_y", pairs, W, torch.float32, max_rows=most)
-        ops.moe_gemm(act, self.w_down, y, tiles, None, None if on_input else src_scale)
+        ops.moe_gemm(act, self.w_down, y, tiles, None, None if on_input else src_scale, matrix_cores=rt.tuned)
         shared = None
         if self.shared_size is not None:
             sact = rt.buffer("moe_shared_act", n, self.shared_size)

@@ -158,7 +158,7 @@ def test_latent_attention_alone(dtype, H, D, Dv, Rq, R, scale):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,D,Dv,cap", [(2, 12, 20, 8.0), (1, 20, 70, 15.0), (3, 4, 6, 2.0), (1, 100, 33, 30.0)])
+@pytest.mark.parametrize("H,D,Dv,cap", [(2, 12, 20, 8.0), (1, 20, 70, 15.0), (3, 4, 6, 2.0), (1, 100, 33, 30.0), (1, 300, 17, 12.0)])
 def test_mlstm_alone(dtype, H, D, Dv, cap):
     from flambeau_amd.parts import MIXERS, PartSpec
     rt = make_rt(dtype)
@@ -177,10 +177,10 @@ def test_mlstm_alone(dtype, H, D, Dv, cap):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n", [1, 7, 150])
-def test_feed_forwards_alone(dtype, n):
+@pytest.mark.parametrize("W", [40, 64])          # 64: in bfloat16 the experts' products run on the matrix cores
+def test_feed_forwards_alone(dtype, n, W):
     from flambeau_amd.parts import FEED_FORWARDS, PartSpec, Product
     rt = make_rt(dtype)
-    W = 40
     x = (torch.randn(n, W, generator=torch.Generator().manual_seed(n))).to(TORCH[dtype])
     xs = x.double().numpy()
     tol = 3e-5 if dtype == "float32" else 3e-2
@@ -193,7 +193,7 @@ def test_feed_forwards_alone(dtype, n):
         want = fn(xs @ plain["m.up"].T) @ plain["m.down"].T
         assert np.abs(run(part) - want).max() < tol * np.abs(want).max(), act
     for E, top, shared in ((5, 2, 24), (3, 3, None), (7, 1, 8), (70, 4, None)):
-        spec = dict(hidden_size=W, n_experts=E, top=top, expert_size=16, shared_size=shared)
+        spec = dict(hidden_size=W, n_experts=E, top=top, expert_size=16 if W == 40 else 32, shared_size=shared)
         part, plain = bound_part(FEED_FORWARDS, PartSpec("routed_experts", spec), dtype, rt, seed=E, scale=0.4)
         mlp = {"router": {"experts": E, "top": top}, "shared": {"ff": shared} if shared else None}
         want = pk.moe_ff(xs, plain, "m.", mlp)
@@ -360,3 +360,37 @@ def test_trace_replay_as_a_program(dirs, tmp_path, dtype):
     got = rh.run_program(d, dtype, steps, tmp_path / "o", rh.peak_tokens(steps), 130, extra=("--poison-cache",), stats=stats)
     assert stats["handed_out"] > stats["pool"]
     close(got, ref, dtype, "trace_run")
+
+
+@pytest.mark.parametrize("splits", [2, 8, 64])
+def test_keys_dealt_out_to_several_waves(splits):
+    """The matrix-core attention kernel with every token's keys in several parts (what a decode step behind
+    a long context does) against the same kernel in one part, rows of unequal contexts side by side, some
+    shorter than the number of parts."""
+    from flambeau_amd.cache.storage import CacheStorage
+    from flambeau_amd.kernels import latent_attention as la
+    from flambeau_amd.parts import PagedRowSpec
+    H, R, ps, n_pages = 20, 96, 16, 80
+    store = CacheStorage([PagedRowSpec(R)], [None], torch.device(DEV), torch.bfloat16, n_pages=n_pages, page_size=ps, max_slots=4)
+    pool = store.pools[0]                       # [entries, pages, 2, page, R]: rows, and the same rows transposed
+    pool[:, :, 0].normal_(0.0, 1.0)
+    pool[:, :, 1] = pool[:, :, 0].transpose(-1, -2).reshape(pool[:, :, 1].shape)
+    seqs = [(700, 1), (0, 1), (130, 3), (63, 2)]
+    step = make_step(seqs, ps, n_pages)
+    n = step.n_tokens
+    qa = (torch.randn(n, H * R, generator=torch.Generator().manual_seed(1)) * 0.3).to(torch.bfloat16).to(DEV)
+    cache = store.entries[0].kv
+    one = torch.empty(n, H * R, dtype=torch.float32, device=DEV)
+    la.latent_attention_mfma(qa, one, cache, step.positions, step.tok_seq, step.block_tables[0], H, 0.5)
+    rows = n * 2 * splits * 16
+    part_o = torch.full((rows, R), float("nan"), dtype=torch.float32, device=DEV)
+    part_ml = torch.full((rows, 2), float("nan"), dtype=torch.float32, device=DEV)
+    many = torch.empty_like(one)
+    la.latent_attention_mfma(qa, many, cache, step.positions, step.tok_seq, step.block_tables[0], H, 0.5, 0, splits, part_o, part_ml)
+    assert torch.isfinite(many).all()
+    assert (many - one).abs().max().item() < 2e-3 * one.abs().max().item()
+    # and both against the float kernel
+    plain = torch.empty_like(one)
+    from flambeau_amd.kernels import ops
+    ops.latent_attention(qa.float(), plain, cache, step.positions, step.tok_seq, step.block_tables[0], H, 0.5)
+    assert (one - plain).abs().max().item() < 2e-2 * plain.abs().max().item()
