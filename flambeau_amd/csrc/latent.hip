@@ -191,6 +191,7 @@ __global__ __launch_bounds__(64 * LA_WAVES) void latent_attention_kernel(
             for (int j = 0; j < cnt; ++j) {
                 const int tj = t0 + j;
                 const int page = table[tj / page_size];
+                if (page < 0 || page >= n_pages) continue;          // (rows that pad a batch of fixed shape have no pages)
                 const T* row = pool + ((size_t)page * 2 * page_size + tj % page_size) * R;
                 const float w = ps[j];
 #pragma unroll

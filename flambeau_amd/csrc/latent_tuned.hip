@@ -179,19 +179,19 @@ __global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restri
     if (unit >= total) return;
     const int token = unit / H, h = unit - token * H;
     const size_t base = ((size_t)(token * groups + (h >> 4)) * n_split) * 16 + (h & 15);        // part 0; parts are 16 rows apart
-    float M = -INFINITY;
-    for (int s = 0; s < n_split; ++s) M = fmaxf(M, part_ml[(base + (size_t)s * 16) * 2]);
-    float L = 0.f;
-    for (int s = 0; s < n_split; ++s) {
-        const float ms = part_ml[(base + (size_t)s * 16) * 2];
-        if (ms > -INFINITY) L += part_ml[(base + (size_t)s * 16) * 2 + 1] * expf(ms - M);
-    }
+    // the parts' weights exp(m_s - M) once per wave (lane s holds part s; at most 64 parts), then every dim is a
+    // sum of independent loads
+    const float ms = lane < n_split ? part_ml[(base + (size_t)lane * 16) * 2] : -INFINITY;
+    const float ls = lane < n_split ? part_ml[(base + (size_t)lane * 16) * 2 + 1] : 0.f;
+    const float M = wave_max(ms);
+    const float ws = ms > -INFINITY ? expf(ms - M) : 0.f;
+    const float L = wave_sum(ls * ws);
     const float inv = L > 0.f ? 1.0f / L : 0.f;
     for (int d = lane; d < R; d += 64) {
         float acc = 0.f;
         for (int s = 0; s < n_split; ++s) {
-            const float ms = part_ml[(base + (size_t)s * 16) * 2];
-            if (ms > -INFINITY) acc += part_o[(base + (size_t)s * 16) * R + d] * expf(ms - M);
+            const float w = __shfl(ws, s, FL_WAVE);
+            if (w > 0.f) acc = fmaf(part_o[(base + (size_t)s * 16) * R + d], w, acc);
         }
         z[(size_t)unit * R + d] = acc * inv;
     }
@@ -207,7 +207,7 @@ extern "C" int fl_latent_attention_mfma(const void* qa, float* z, const void* po
                                         int page_size, int n_pages, float scale, int window, int n_split, float* part_o,
                                         float* part_ml, hipStream_t stream) {
     FL_CHECK(n >= 0 && H > 0 && n_pages > 0 && max_blocks > 0, "latent_attention_mfma: bad sizes");
-    FL_CHECK(n_split >= 1 && (n_split == 1 || (part_o && part_ml)), "latent_attention_mfma: %d parts of the keys need a workspace", n_split);
+    FL_CHECK(n_split >= 1 && n_split <= 64 && (n_split == 1 || (part_o && part_ml)), "latent_attention_mfma: %d parts of the keys (at most 64) need a workspace", n_split);
     FL_CHECK(fl_latent_attention_mfma_takes(R, page_size), "latent_attention_mfma: rows of %d values in pages of %d are not taken", R, page_size);
     FL_CHECK((uintptr_t)qa % 16 == 0 && (uintptr_t)pool % 16 == 0 && (uintptr_t)z % 16 == 0, "latent_attention_mfma: operands must be 16-byte aligned");
     FL_CHECK(window >= 0, "latent_attention_mfma: negative window");
@@ -245,9 +245,12 @@ FL_RECORDABLE(fl_latent_attention_mfma)
 template <typename TX, typename TOut, int NS>
 __global__ __launch_bounds__(64 * LT_WAVES) void heads_matmul_mfma_kernel(
     const TX* __restrict__ x, int ldx, const bf16_t* __restrict__ w, TOut* __restrict__ out, int n, int H, int K, int J,
-    const float* __restrict__ gate, int ldg, int gate_col0) {
+    const float* __restrict__ gate, int ldg, int gate_col0, int j_parts) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int t0 = (blockIdx.x * LT_WAVES + wave) * 16, h = blockIdx.y;
+    // a wave takes 16 tokens and every j_parts-th tile of 16 output columns (few tokens: many parts, so that
+    // a decode step still fills the chip)
+    const int unit = blockIdx.x * LT_WAVES + wave;
+    const int t0 = (unit / j_parts) * 16, j_first = unit % j_parts, h = blockIdx.y;
     if (t0 >= n) return;
     const int col = lane & 15, g = lane >> 4;
     const int ns = K >> 5;
@@ -263,7 +266,7 @@ __global__ __launch_bounds__(64 * LT_WAVES) void heads_matmul_mfma_kernel(
     }
     const float gv = (gate && live) ? 1.0f / (1.0f + expf(-gate[(size_t)token * ldg + gate_col0 + h])) : 1.0f;
     const bf16_t* wh = w + (size_t)h * J * K;
-    for (int jt = 0; jt < J / 16; ++jt) {
+    for (int jt = j_first; jt < J / 16; jt += j_parts) {
         f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
         const bf16_t* row = wh + (size_t)(16 * jt + col) * K + 8 * g;
 #pragma unroll
@@ -287,9 +290,13 @@ extern "C" int fl_heads_matmul_mfma(const void* x, int x_dtype, int ldx, const v
     FL_CHECK(!gate || ldg >= gate_col0 + H, "heads_matmul_mfma: gate columns beyond rows %d wide", ldg);
     if (n == 0) return 0;
     FL_CHECK(H <= 65535, "heads_matmul_mfma: too many heads");
-    dim3 grid(ceil_div(n, 16 * LT_WAVES), H);
+    // enough waves for four per compute unit, as far as the column tiles go
+    const int groups = ceil_div(n, 16);
+    int j_parts = (4 * fl_units()) / (groups * H);
+    j_parts = j_parts < 1 ? 1 : (j_parts > J / 16 ? J / 16 : j_parts);
+    dim3 grid(ceil_div(groups * j_parts, LT_WAVES), H);
     const int ns = K / 32;
-#define FL_HMM(TX, TO, NS) heads_matmul_mfma_kernel<TX, TO, NS><<<grid, 64 * LT_WAVES, 0, stream>>>((const TX*)x, ldx, (const bf16_t*)w, (TO*)out, n, H, K, J, gate, ldg, gate_col0)
+#define FL_HMM(TX, TO, NS) heads_matmul_mfma_kernel<TX, TO, NS><<<grid, 64 * LT_WAVES, 0, stream>>>((const TX*)x, ldx, (const bf16_t*)w, (TO*)out, n, H, K, J, gate, ldg, gate_col0, j_parts)
 #define FL_HMM_NS(TX, TO)                      \
     do {                                       \
         if (ns <= 2) FL_HMM(TX, TO, 2);        \

@@ -47,6 +47,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[a][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
     const bf16x8 zero = {(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
+#pragma unroll 4
     for (int k0 = 0; k0 < K; k0 += 32) {
         bf16x8 av[2], bv[4];
 #pragma unroll

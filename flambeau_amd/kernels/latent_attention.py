@@ -45,7 +45,7 @@ class PlainLatentAttention:
 
 
 SPLIT_TARGET_WAVES = 1024     # four per compute unit
-SPLIT_MIN_KEYS = 128          # a part of the keys is at least two chunks of 64
+SPLIT_MIN_KEYS = 64           # a part of the keys is at least one chunk of 64
 
 
 def key_splits(batch, n_heads: int) -> int:

@@ -66,6 +66,11 @@ CONFIGS = {
         (_rec(2, 32, 32, 10.0), _dense(64)),
         (_att(4, 64, 48, 32, 96, 0.3), None),
     ], loop=(0, 1, 2)), seed=31, std=0.15, page_size=16),
+    # attention layers only: no mixer advances a state, so steps of single tokens replay captured graphs
+    "T": dict(config=_model(90, 64, 1e-5, [
+        (_att(4, 32, 16, 16, 32, 0.6), _moe(3, 1, 32, 16)),
+        (_att(3, 8, 24, 12, 20, 0.9), _dense(48)),
+    ], loop=(1, 2, 2)), seed=41, std=0.15, page_size=16),
 }
 
 STORE = {"float32": torch.float32, "bfloat16": torch.bfloat16}

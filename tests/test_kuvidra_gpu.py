@@ -238,7 +238,8 @@ def test_the_stream_after_every_layer(dirs, name, dtype):
 
 # ---------------------------------------------------------------- whole models in every cutting
 LENGTHS = {"P": [40, 70, 97, 1, 33, 64, 2, 90, 55, 128, 21], "Q": [97, 1, 150, 64, 31, 2, 120, 17, 65],
-           "R": [33, 80, 5, 129, 64, 16, 100], "S": [150, 64, 3, 65, 1, 200, 31, 90]}
+           "R": [33, 80, 5, 129, 64, 16, 100], "S": [150, 64, 3, 65, 1, 200, 31, 90],
+           "T": [40, 100, 7, 64, 130, 2, 55]}
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -257,6 +258,30 @@ def test_every_cutting(dirs, name, dtype):
         assert sum(p.n_acquired for p in pools) > sum(p.n_pages for p in pools), mode       # pages were used again
         assert not runner.manager.live and runner.manager.n_free_slots == 4
         close(got, ref, dtype, f"{name} {mode}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_single_tokens_replay_graphs_where_no_state_is_advanced(dirs, dtype):
+    """A model of attention layers alone captures its decode steps (padded to a bucket: rows without pages
+    ride along); one with an mLSTM layer never does.  Both give the plain logits."""
+    from flambeau_amd.engine import StepEntry
+    d = dirs[("T", dtype)]
+    reqs = rh.make_requests(90, [20, 33, 5], seed=12)
+    ref = reference(d, reqs)
+    runner = runner_for(d, dtype, n_pages=24, page_size=16, max_tokens=256)
+    assert runner.decode_graphs
+    assert not runner_for(dirs[("P", dtype)], dtype, n_pages=24, page_size=8).decode_graphs
+    got = {}
+    for rid, toks in reqs.items():
+        assert runner.begin(rid)
+        runner.step([StepEntry(rid, toks[:3], [])])
+    for i in range(3, 33):
+        live = [rid for rid, toks in reqs.items() if i < len(toks)]
+        rows = runner.step([StepEntry(rid, [reqs[rid][i]], [0]) for rid in live]).cpu().double().numpy()
+        for rid, row in zip(live, rows):
+            got[(rid, i)] = row
+    assert runner._graphs
+    close(got, ref, dtype, "graphs")
 
 
 def test_a_batch_equals_each_request_alone(dirs):
