@@ -103,9 +103,10 @@ int fl_moe_route(const float* logits, int ld, int col0, int n, int E, int top, i
 int fl_moe_tile_rows(void);
 int fl_moe_gemm(const void* x, int dtype, const int* src_row, const float* src_scale, const void* w,
                 float* out, const int* tiles, int max_tiles, int N, int K, hipStream_t stream);
-// fl_moe_gemm on the matrix cores (bfloat16 x and w; moe_tuned.hip)
+// fl_moe_gemm on the matrix cores (bfloat16 x and w; moe_tuned.hip); n_rows: the sorted pairs of the step (few: the
+// form that only streams the weights)
 int fl_moe_gemm_mfma(const void* x, const int* src_row, const float* src_scale, const void* w, float* out,
-                     const int* tiles, int max_tiles, int N, int K, hipStream_t stream);
+                     const int* tiles, int max_tiles, int n_rows, int N, int K, hipStream_t stream);
 int fl_moe_gemm_mfma_takes(int N, int K);
 // out[m][f] = sum_k x[m][k] w[f][k] for few features f: one wave per output, float sums in a fixed order
 int fl_gemm_few(const void* x, const void* w, float* out, int dtype, int M, int N, int K, hipStream_t stream);

@@ -47,9 +47,13 @@ __global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_mfma_kernel(
     const size_t page_stride = (size_t)2 * page_size * R;
     const bool head_live = h0 + col < H;
 
-    // the folded queries of this lane's head, scaled: B operand of every score product
-    bf16x8 qreg[NS];
+    // the folded queries of this lane's head, scaled: B operand of every score product.  They wait in LDS, each lane's
+    // own 16 bytes per step (written and read by the same lane: no barrier, no bank conflict), which leaves the
+    // registers to the accumulators and to loads in flight.
+    __shared__ bf16x8 qs[LT_WAVES][NS * 64];
+    bf16x8* qmine = &qs[wave][lane];
     {
+        bf16x8 qreg[NS];
         const bf16_t* qr = qa + ((size_t)token * H + h0 + (head_live ? col : 0)) * R;
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
@@ -61,6 +65,7 @@ __global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_mfma_kernel(
 #pragma unroll
                 for (int e = 0; e < 8; ++e) qreg[s][e] = (bf16_t)0.f;
             }
+            qmine[s * 64] = qreg[s];
         }
     }
     f32x4 o[2 * NS];                                               // Z^T tiles: dims 16 t + 4 g + r of head `col`
@@ -89,7 +94,7 @@ __global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_mfma_kernel(
             const bf16_t* row = pool + (size_t)page * page_stride + (size_t)(kc % page_size) * R + 8 * g;
 #pragma unroll
             for (int s = 0; s < NS; ++s)
-                if (s < ns) sacc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(row + 32 * s), qreg[s], sacc[a], 0, 0, 0);
+                if (s < ns) sacc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(row + 32 * s), qmine[s * 64], sacc[a], 0, 0, 0);
         }
         // lane (head col, g): sacc[2 q + b][e] is key t0 + 32 q + 8 g + 4 b + e
         float cmax = -INFINITY;
@@ -189,10 +194,9 @@ __global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restri
     const float inv = L > 0.f ? 1.0f / L : 0.f;
     for (int d = lane; d < R; d += 64) {
         float acc = 0.f;
-        for (int s = 0; s < n_split; ++s) {
-            const float w = __shfl(ws, s, FL_WAVE);
-            if (w > 0.f) acc = fmaf(part_o[(base + (size_t)s * 16) * R + d], w, acc);
-        }
+#pragma unroll 8
+        for (int s = 0; s < n_split; ++s)              // (an empty part left zeros and has weight 0)
+            acc = fmaf(part_o[(base + (size_t)s * 16) * R + d], __shfl(ws, s, FL_WAVE), acc);
         z[(size_t)unit * R + d] = acc * inv;
     }
 }

@@ -4,13 +4,112 @@
 #include "recordable.h"
 
 #define MT_TILE 64            // rows of a tile (fl_moe_route cuts the sorted pairs into tiles of this many)
-#define MT_FEATURES 128       // output features per block: four waves of 32
+#define MT_FEATURES 256       // output features per block: four waves of 64
 
 // out[p][:] = (scale[p] * x[src[p]]) W_e^T over the tiles of fl_moe_route, as fl_moe_gemm computes it, with
+// v_mfma_f32_16x16x32_bf16, K in steps of 32.  A wave takes 64 features (four A operands, read straight
+// from the expert's rows, a step ahead) against the tile's rows in groups of 16 (B operands).  The rows
+// are gathered, scaled and rounded once per block and shared through LDS (two slots, one barrier a
+// step; the 16-byte pieces of a row are exchanged by (row / 2) % 4 so that the reads of a group of
+// rows meet in no bank).  Row groups a tile does not have are skipped, so a decode step (a row or two
+// per expert) streams the weights once.
+__global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __restrict__ x, const int* __restrict__ src_row,
+                                                            const float* __restrict__ src_scale, const bf16_t* __restrict__ w,
+                                                            float* __restrict__ out, const int* __restrict__ tiles, int N, int K) {
+    __shared__ bf16x8 xs[2][MT_TILE * 4];
+    const int e = tiles[4 * blockIdx.y + 0];
+    if (e < 0) return;                                   // (the whole block: tiles are per block)
+    const int p0 = tiles[4 * blockIdx.y + 1], M = tiles[4 * blockIdx.y + 2];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int col = lane & 15, g = lane >> 4;
+    const int f0 = blockIdx.x * MT_FEATURES + wave * 64;
+    const bf16_t* we = w + (size_t)e * N * K;
+    const bf16_t* wrow[4];
+    bool wlive[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        const int f = f0 + 16 * a + col;
+        wlive[a] = f < N;
+        wrow[a] = we + (size_t)(wlive[a] ? f : 0) * K + 8 * g;
+    }
+    const int groups = (M + 15) >> 4;
+    // this thread's share of the rows' staging: row threadIdx.x / 4, the 16-byte piece threadIdx.x % 4 of a step
+    const int srow = threadIdx.x >> 2, spiece = threadIdx.x & 3;
+    const bool slive = srow < M;
+    const int sp = p0 + (slive ? srow : 0);
+    const bf16_t* sx = x + (size_t)(src_row ? src_row[sp] : sp) * K + 8 * spiece;
+    const float sscale = src_scale ? src_scale[sp] : 1.0f;
+    const int sslot = srow * 4 + (spiece ^ ((srow >> 1) & 3));
+    const bf16x8 zero = {(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
+    auto staged = [&](int k0) {
+        bf16x8 v = slive ? *(const bf16x8*)(sx + k0) : zero;
+        if (src_scale) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = (bf16_t)((float)v[i] * sscale);
+        }
+        return v;
+    };
+    f32x4 acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[a][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    bf16x8 av[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) av[a] = wlive[a] ? *(const bf16x8*)(wrow[a]) : zero;
+    xs[0][sslot] = staged(0);
+    __syncthreads();
+    int cur = 0;
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const bool more = k0 + 32 < K;
+        bf16x8 an[4], xn = zero;
+        if (more) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) an[a] = wlive[a] ? *(const bf16x8*)(wrow[a] + k0 + 32) : zero;
+            xn = staged(k0 + 32);
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (t < groups) {
+                const int r = 16 * t + col;
+                const bf16x8 bv = xs[cur][r * 4 + (g ^ ((r >> 1) & 3))];
+#pragma unroll
+                for (int a = 0; a < 4; ++a) acc[a][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[a], bv, acc[a][t], 0, 0, 0);
+            }
+        if (more) {
+            xs[cur ^ 1][sslot] = xn;
+#pragma unroll
+            for (int a = 0; a < 4; ++a) av[a] = an[a];
+        }
+        __syncthreads();
+        cur ^= 1;
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int r = 16 * t + col;
+        if (r >= M) continue;
+        float* dst = out + (size_t)(p0 + r) * N;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const int f = f0 + 16 * a + 4 * g;
+            if (f + 3 < N) {
+                *(f32x4*)(dst + f) = acc[a][t];
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (f + q < N) dst[f + q] = acc[a][t][q];
+            }
+        }
+    }
+}
+
+#define MT_STREAM_FEATURES 128       // output features per block of the streaming form: four waves of 32
+// The same for steps of few rows (decoding), where nearly every tile holds a row or two and all a block
+// does is stream its expert's weights: no LDS, no barrier.  out[p][:] = (scale[p] * x[src[p]]) W_e^T with
 // v_mfma_f32_16x16x32_bf16: a wave takes 32 features (two A operands, read straight from the expert's
 // rows) against up to four groups of 16 rows (B operands); K in steps of 32.  Row groups a tile does not
 // have are skipped, so a decode step (a row or two per expert) streams the weights once.
-__global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __restrict__ x, const int* __restrict__ src_row,
+__global__ __launch_bounds__(256) void moe_gemm_mfma_stream_kernel(const bf16_t* __restrict__ x, const int* __restrict__ src_row,
                                                             const float* __restrict__ src_scale, const bf16_t* __restrict__ w,
                                                             float* __restrict__ out, const int* __restrict__ tiles, int N, int K) {
     const int e = tiles[4 * blockIdx.y + 0];
@@ -18,7 +117,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
     const int p0 = tiles[4 * blockIdx.y + 1], M = tiles[4 * blockIdx.y + 2];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int col = lane & 15, g = lane >> 4;
-    const int f0 = blockIdx.x * MT_FEATURES + wave * 32;
+    const int f0 = blockIdx.x * MT_STREAM_FEATURES + wave * 32;
     if (f0 >= N) return;
     const bf16_t* we = w + (size_t)e * N * K;
     const bf16_t* wrow[2];
@@ -90,13 +189,18 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
 extern "C" int fl_moe_gemm_mfma_takes(int N, int K) { return N > 0 && N % 4 == 0 && K > 0 && K % 32 == 0; }
 
 extern "C" int fl_moe_gemm_mfma(const void* x, const int* src_row, const float* src_scale, const void* w, float* out,
-                                const int* tiles, int max_tiles, int N, int K, hipStream_t stream) {
-    FL_CHECK(max_tiles >= 0 && fl_moe_gemm_mfma_takes(N, K), "moe_gemm_mfma: %d features over %d values are not taken", N, K);
+                                const int* tiles, int max_tiles, int n_rows, int N, int K, hipStream_t stream) {
+    FL_CHECK(max_tiles >= 0 && n_rows >= 0 && fl_moe_gemm_mfma_takes(N, K), "moe_gemm_mfma: %d features over %d values are not taken", N, K);
     FL_CHECK((uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0, "moe_gemm_mfma: operands must be 16-byte aligned");
     if (max_tiles == 0) return 0;
     FL_CHECK(max_tiles <= 65535, "moe_gemm_mfma: %d row tiles are more than one grid takes", max_tiles);
-    dim3 grid(ceil_div(N, MT_FEATURES), max_tiles);
-    moe_gemm_mfma_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)x, src_row, src_scale, (const bf16_t*)w, out, tiles, N, K);
+    if (n_rows <= 2 * MT_TILE) {
+        dim3 grid(ceil_div(N, MT_STREAM_FEATURES), max_tiles);
+        moe_gemm_mfma_stream_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)x, src_row, src_scale, (const bf16_t*)w, out, tiles, N, K);
+    } else {
+        dim3 grid(ceil_div(N, MT_FEATURES), max_tiles);
+        moe_gemm_mfma_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)x, src_row, src_scale, (const bf16_t*)w, out, tiles, N, K);
+    }
     FL_LAUNCH_CHECK();
     return 0;
 }

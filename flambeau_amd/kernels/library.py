@@ -42,7 +42,7 @@ _SIGNATURES = {
     "fl_headnorm_gate": [P, P, P, I, I, P, I, I, I, I, F, P],
     "fl_moe_route": [P, I, I, I, I, I, I, I, P, P, P, P, P, I, P],
     "fl_moe_gemm": [P, I, P, P, P, P, P, I, I, I, P],
-    "fl_moe_gemm_mfma": [P, P, P, P, P, P, I, I, I, P],
+    "fl_moe_gemm_mfma": [P, P, P, P, P, P, I, I, I, I, P],
     "fl_gemm_few": [P, P, P, I, I, I, I, P],
     "fl_moe_combine": [P, P, I, P, P, I, I, P, I, I, P],
     "fl_activation": [P, P, I, L, I, P],

@@ -460,7 +460,7 @@ def moe_gemm(x, w, out, tiles, src_row=None, src_scale=None, matrix_cores=False)
                  _check(src_row, "moe_gemm.src_row", torch.int32, (P_,)) if src_row is not None else None,
                  _check(src_scale, "moe_gemm.src_scale", torch.float32, (P_,)) if src_scale is not None else None,
                  _check(w, "moe_gemm.w"), _check(out, "moe_gemm.out", torch.float32, (P_, N)),
-                 _check(tiles, "moe_gemm.tiles", torch.int32, (None, 4)), tiles.shape[0], N, K, stream_handle())
+                 _check(tiles, "moe_gemm.tiles", torch.int32, (None, 4)), tiles.shape[0], P_, N, K, stream_handle())
             return out
     call("fl_moe_gemm", _check(x, "moe_gemm.x", w.dtype, (None, K)), dtype_code(w.dtype),
          _check(src_row, "moe_gemm.src_row", torch.int32, (P_,)) if src_row is not None else None,
