@@ -47,13 +47,9 @@ __global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_mfma_kernel(
     const size_t page_stride = (size_t)2 * page_size * R;
     const bool head_live = h0 + col < H;
 
-    // the folded queries of this lane's head, scaled: B operand of every score product.  They wait in LDS, each lane's
-    // own 16 bytes per step (written and read by the same lane: no barrier, no bank conflict), which leaves the
-    // registers to the accumulators and to loads in flight.
-    __shared__ bf16x8 qs[LT_WAVES][NS * 64];
-    bf16x8* qmine = &qs[wave][lane];
+    // the folded queries of this lane's head, scaled: B operand of every score product
+    bf16x8 qreg[NS];
     {
-        bf16x8 qreg[NS];
         const bf16_t* qr = qa + ((size_t)token * H + h0 + (head_live ? col : 0)) * R;
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
@@ -65,7 +61,6 @@ __global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_mfma_kernel(
 #pragma unroll
                 for (int e = 0; e < 8; ++e) qreg[s][e] = (bf16_t)0.f;
             }
-            qmine[s * 64] = qreg[s];
         }
     }
     f32x4 o[2 * NS];                                               // Z^T tiles: dims 16 t + 4 g + r of head `col`
@@ -94,7 +89,7 @@ __global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_mfma_kernel(
             const bf16_t* row = pool + (size_t)page * page_stride + (size_t)(kc % page_size) * R + 8 * g;
 #pragma unroll
             for (int s = 0; s < NS; ++s)
-                if (s < ns) sacc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(row + 32 * s), qmine[s * 64], sacc[a], 0, 0, 0);
+                if (s < ns) sacc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(row + 32 * s), qreg[s], sacc[a], 0, 0, 0);
         }
         // lane (head col, g): sacc[2 q + b][e] is key t0 + 32 q + 8 g + 4 b + e
         float cmax = -INFINITY;
@@ -177,28 +172,31 @@ __global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_mfma_kernel(
 }
 
 // z[token][head][:] = sum_s o_s exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s, over the parts of the keys
-// (rising s; an empty part has m = -inf and adds nothing).  One wave per (token, head).
+// (rising s; an empty part left zeros and has weight 0).  A block takes 256 dims of one (token, head): its
+// first wave makes the parts' weights, then every thread adds its dim's parts, all loads independent.
 __global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                           float* __restrict__ z, int total, int H, int R, int groups, int n_split) {
-    const int unit = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-    if (unit >= total) return;
+                                                           float* __restrict__ z, int H, int R, int groups, int n_split) {
+    __shared__ float ws[64];
+    __shared__ float inv_l;
+    const int unit = blockIdx.x, d = blockIdx.y * 256 + threadIdx.x;
     const int token = unit / H, h = unit - token * H;
     const size_t base = ((size_t)(token * groups + (h >> 4)) * n_split) * 16 + (h & 15);        // part 0; parts are 16 rows apart
-    // the parts' weights exp(m_s - M) once per wave (lane s holds part s; at most 64 parts), then every dim is a
-    // sum of independent loads
-    const float ms = lane < n_split ? part_ml[(base + (size_t)lane * 16) * 2] : -INFINITY;
-    const float ls = lane < n_split ? part_ml[(base + (size_t)lane * 16) * 2 + 1] : 0.f;
-    const float M = wave_max(ms);
-    const float ws = ms > -INFINITY ? expf(ms - M) : 0.f;
-    const float L = wave_sum(ls * ws);
-    const float inv = L > 0.f ? 1.0f / L : 0.f;
-    for (int d = lane; d < R; d += 64) {
-        float acc = 0.f;
-#pragma unroll 8
-        for (int s = 0; s < n_split; ++s)              // (an empty part left zeros and has weight 0)
-            acc = fmaf(part_o[(base + (size_t)s * 16) * R + d], __shfl(ws, s, FL_WAVE), acc);
-        z[(size_t)unit * R + d] = acc * inv;
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        const float ms = lane < n_split ? part_ml[(base + (size_t)lane * 16) * 2] : -INFINITY;
+        const float ls = lane < n_split ? part_ml[(base + (size_t)lane * 16) * 2 + 1] : 0.f;
+        const float M = wave_max(ms);
+        const float w = ms > -INFINITY ? expf(ms - M) : 0.f;
+        const float L = wave_sum(ls * w);
+        ws[lane] = w;
+        if (lane == 0) inv_l = L > 0.f ? 1.0f / L : 0.f;
     }
+    __syncthreads();
+    if (d >= R) return;
+    float acc = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < n_split; ++s) acc = fmaf(part_o[(base + (size_t)s * 16) * R + d], ws[s], acc);
+    z[(size_t)unit * R + d] = acc * inv_l;
 }
 
 // Whether the kernel takes a pool's shape: rows of a multiple of 32 values up to 512, pages of a multiple of 16 rows.
@@ -233,13 +231,205 @@ extern "C" int fl_latent_attention_mfma(const void* qa, float* z, const void* po
 #undef FL_LT
     FL_LAUNCH_CHECK();
     if (n_split > 1) {
-        const int total = n * H;
-        latent_merge_kernel<<<(total + 3) / 4, 256, 0, stream>>>(part_o, part_ml, z, total, H, R, groups, n_split);
+        dim3 mgrid(n * H, ceil_div(R, 256));
+        latent_merge_kernel<<<mgrid, 256, 0, stream>>>(part_o, part_ml, z, H, R, groups, n_split);
         FL_LAUNCH_CHECK();
     }
     return 0;
 }
 FL_RECORDABLE(fl_latent_attention_mfma)
+
+
+// The same walk for prompt portions, four waves to a block that share their keys: a tile (from the host:
+// first token, tokens, first group of 16 heads, groups; tokens x groups <= 4, all of one request) loads
+// every chunk of 64 rows once into LDS, as it is and transposed, and its waves read their operands from
+// there.  Without this every wave fetches every row itself and the kernel runs at the rate of the
+// caches, 16 flops a byte.  Rows are padded by 16 bytes so that the 16 rows (or dims) of an operand
+// start in different banks.  A wave whose token lies before a chunk sits the chunk out.
+template <int NS>
+__global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_shared_kernel(
+    const bf16_t* __restrict__ qa, float* __restrict__ z, const bf16_t* __restrict__ pool,
+    const int* __restrict__ positions, const int* __restrict__ tok_seq, const int* __restrict__ block_table,
+    int max_blocks, int H, int R, int page_size, int n_pages, float scale, int window, const int* __restrict__ tiles) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lt_smem[];
+    const int stride_r = R + 8, stride_c = LT_CHUNK + 8;
+    bf16_t* ks = (bf16_t*)lt_smem;                                  // [64 keys][R + 8]
+    bf16_t* vs = ks + (size_t)LT_CHUNK * stride_r;                  // [R dims][64 + 8]
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int t_first = tiles[4 * blockIdx.x], n_tok = tiles[4 * blockIdx.x + 1];
+    const int g_first = tiles[4 * blockIdx.x + 2], n_grp = tiles[4 * blockIdx.x + 3];
+    const int tw = wave / n_grp, gw = wave - tw * n_grp;
+    const bool active = tw < n_tok;
+    const int token = t_first + (active ? tw : 0), h0 = (g_first + gw) * 16;
+    const int col = lane & 15, g = lane >> 4;
+    const int ns = R >> 5;
+    const int p = active ? positions[token] : -1;
+    const int p_max = positions[t_first + n_tok - 1];              // a request's tokens of a step stand in rising order
+    const int* table = block_table + (size_t)tok_seq[t_first] * max_blocks;
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const int lo_min = window > 0 ? max(0, positions[t_first] - window + 1) : 0;
+    const size_t page_stride = (size_t)2 * page_size * R;
+    const bool head_live = active && h0 + col < H;
+    bf16x8 qreg[NS];
+    {
+        const bf16_t* qr = qa + ((size_t)token * H + (head_live ? h0 + col : 0)) * R;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            if (s < ns && head_live) {
+                const bf16x8 v = *(const bf16x8*)(qr + 32 * s + 8 * g);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qreg[s][e] = (bf16_t)((float)v[e] * scale);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qreg[s][e] = (bf16_t)0.f;
+            }
+        }
+    }
+    f32x4 o[2 * NS];
+#pragma unroll
+    for (int t = 0; t < 2 * NS; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    const int pieces_r = R >> 3;                                    // 16-byte pieces of a row
+    for (int t0 = lo_min & ~(LT_CHUNK - 1); t0 <= p_max; t0 += LT_CHUNK) {
+        // ---- the chunk into LDS: rows as they are, and the pages' transposed copies dim by dim.  The pages of the
+        // chunk's four runs of 16 keys are looked up first (pages hold a multiple of 16 rows), so that all copies
+        // of a thread are in flight at once; a run beyond the newest token takes that token's page and is masked.
+        const bf16_t* run_rows[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int kc = min(t0 + 16 * j, p_max & ~15);
+            int page = table[kc / page_size];
+            page = min(max(page, 0), n_pages - 1);
+            run_rows[j] = pool + (size_t)page * page_stride + (size_t)(kc % page_size) * R;       // row kc of the page; its transposed copy lies page_size * R further, at column kc % page_size
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {                             // wave w copies rows w, w + 4, ...: row 4 i + w lies in run i / 4
+            const int row = 4 * i + wave;
+            const bf16_t* src = run_rows[i >> 2] + (size_t)(row & 15) * R;
+            for (int c = lane; c < pieces_r; c += 64) *(bf16x8*)(ks + (size_t)row * stride_r + 8 * c) = *(const bf16x8*)(src + 8 * c);
+        }
+        {
+            const int k8 = threadIdx.x & 7;                        // this thread's 8 keys of every dim: run k8 / 2, its first or second half
+            const int kc = min(t0 + 16 * (k8 >> 1), p_max & ~15);
+            const bf16_t* src = run_rows[0];
+#pragma unroll
+            for (int j = 1; j < 4; ++j) src = (k8 >> 1) == j ? run_rows[j] : src;
+            src += (size_t)(page_size - (kc % page_size)) * R + (kc % page_size) + 8 * (k8 & 1);    // from row kc of the page to column kc (+ 8) of its transposed copy
+            for (int dim = threadIdx.x >> 3; dim < R; dim += 32)
+                *(bf16x8*)(vs + (size_t)dim * stride_c + 8 * k8) = *(const bf16x8*)(src + (size_t)dim * page_size);
+        }
+        __syncthreads();
+        if (active && t0 <= p && t0 + LT_CHUNK - 1 >= lo) {
+            f32x4 sacc[4];
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                sacc[a] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                const bf16_t* row = ks + (size_t)(32 * (a >> 1) + 8 * (col >> 2) + 4 * (a & 1) + (col & 3)) * stride_r + 8 * g;
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+                    if (s < ns) sacc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(row + 32 * s), qreg[s], sacc[a], 0, 0, 0);
+            }
+            float cmax = -INFINITY;
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int key = t0 + 32 * (a >> 1) + 8 * g + 4 * (a & 1) + e;
+                    if (key > p || key < lo) sacc[a][e] = -INFINITY;
+                    cmax = fmaxf(cmax, sacc[a][e]);
+                }
+            cmax = fmaxf(cmax, __shfl_xor(cmax, 16, FL_WAVE));
+            cmax = fmaxf(cmax, __shfl_xor(cmax, 32, FL_WAVE));
+            // The base of the exponents follows the maximum lazily: it moves only when a score exceeds it by more
+            // than 8 (weights stay below e^8, exact enough in bfloat16 and float), so that in most chunks nothing
+            // is rescaled and the sums can stay where the matrix cores accumulate them.
+            const float m_new = (cmax > m + 8.0f) ? cmax : m;      // finite after the first chunk: it holds a key this wave sees
+            const bool moved = __any(m_new != m);
+            const float corr = expf(m - m_new);
+            m = m_new;
+            bf16x8 pb[2];
+            float lsum = 0.f;
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const bf16_t w = (bf16_t)expf(sacc[a][e] - m_new);
+                    pb[a >> 1][4 * (a & 1) + e] = w;
+                    lsum += (float)w;
+                }
+            lsum += __shfl_xor(lsum, 16, FL_WAVE);
+            lsum += __shfl_xor(lsum, 32, FL_WAVE);
+            l = l * corr + lsum;
+            if (moved) {
+#pragma unroll
+                for (int t = 0; t < 2 * NS; ++t)
+                    if (t < 2 * ns) o[t] *= corr;
+            }
+            const bool edge = t0 + LT_CHUNK - 1 > p || t0 < lo;
+#pragma unroll
+            for (int t = 0; t < 2 * NS; ++t) {
+                if (t < 2 * ns) {
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        const int key0 = t0 + 32 * q + 8 * g;
+                        bf16x8 v = *(const bf16x8*)(vs + (size_t)(16 * t + col) * stride_c + 32 * q + 8 * g);
+                        if (edge) {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e)
+                                if (key0 + e > p || key0 + e < lo) v[e] = (bf16_t)0.f;
+                        }
+                        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pb[q], o[t], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (!head_live) return;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    float* zr = z + ((size_t)token * H + h0 + col) * R;
+#pragma unroll
+    for (int t = 0; t < 2 * NS; ++t)
+        if (t < 2 * ns) *(f32x4*)(zr + 16 * t + 4 * g) = o[t] * inv;
+}
+
+extern "C" long fl_latent_attention_shared_lds(int R) { return (long)LT_CHUNK * (R + 8) * 2 + (long)R * (LT_CHUNK + 8) * 2; }
+
+// tiles [n_tiles][4] = (first token, tokens, first group of 16 heads, groups): tokens x groups <= 4, the tokens of one request
+extern "C" int fl_latent_attention_shared(const void* qa, float* z, const void* pool, const int* positions,
+                                          const int* tok_seq, const int* block_table, int max_blocks, int H, int R,
+                                          int page_size, int n_pages, float scale, int window, const int* tiles, int n_tiles,
+                                          hipStream_t stream) {
+    FL_CHECK(n_tiles >= 0 && H > 0 && n_pages > 0 && max_blocks > 0, "latent_attention_shared: bad sizes");
+    FL_CHECK(fl_latent_attention_mfma_takes(R, page_size), "latent_attention_shared: rows of %d values in pages of %d are not taken", R, page_size);
+    FL_CHECK((uintptr_t)qa % 16 == 0 && (uintptr_t)pool % 16 == 0 && (uintptr_t)z % 16 == 0, "latent_attention_shared: operands must be 16-byte aligned");
+    
+    FL_CHECK(window >= 0, "latent_attention_shared: negative window");
+    if (n_tiles == 0) return 0;
+    const size_t lds = (size_t)fl_latent_attention_shared_lds(R);
+    const int ns = R / 32;
+#define FL_LTS(NS)                                                                                                     \
+    do {                                                                                                               \
+        static bool sized = false;                                                                                     \
+        if (!sized) {                                                                                                  \
+            hipError_t e_ = hipFuncSetAttribute((const void*)latent_attention_shared_kernel<NS>,                      \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);              \
+            FL_CHECK(e_ == hipSuccess, "latent_attention_shared: %s", hipGetErrorString(e_));                          \
+            sized = true;                                                                                              \
+        }                                                                                                              \
+        latent_attention_shared_kernel<NS><<<n_tiles, 64 * LT_WAVES, lds, stream>>>(                                  \
+            (const bf16_t*)qa, z, (const bf16_t*)pool, positions, tok_seq, block_table, max_blocks, H, R, page_size,   \
+            n_pages, scale, window, tiles);                                                                            \
+    } while (0)
+    if (ns <= 2) FL_LTS(2);
+    else if (ns <= 4) FL_LTS(4);
+    else if (ns <= 8) FL_LTS(8);
+    else FL_LTS(16);
+#undef FL_LTS
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_latent_attention_shared)
 
 // ------------------------------------------------------------------ one product per head on the matrix cores
 // out[t][h][j] = sum_k x[t][h][k] w[h][j][k]   (x float or bfloat16 rows ldx apart, w bfloat16 [H][J][K], K a multiple

@@ -43,6 +43,10 @@ class PlainLatentAttention:
         """What the kernels decide from the contexts' lengths (part of a recorded step's key)."""
         return ()
 
+    def metadata(self, batch, mixers) -> dict:
+        """Integer arrays the kernels want uploaded with the step (work lists); none here."""
+        return {}
+
 
 SPLIT_TARGET_WAVES = 1024     # four per compute unit
 SPLIT_MIN_KEYS = 64           # a part of the keys is at least one chunk of 64
@@ -57,9 +61,30 @@ def key_splits(batch, n_heads: int) -> int:
     return 1 << (parts.bit_length() - 1)          # a power of two: few different launches while contexts grow
 
 
+def shared_tiles(batch, groups: int):
+    """The blocks of the kernel that shares its keys among four waves: ``[n, 4]`` = (first token, tokens, first
+    group of 16 heads, groups) with tokens x groups <= 4 and all tokens of one request.  The list's length
+    follows from the rows per request alone."""
+    import numpy as np
+    out = []
+    if groups >= 4:
+        for q0, ql in zip(batch.q_starts, batch.q_lens):
+            for t in range(q0, q0 + ql):
+                out += [(t, 1, g0, min(4, groups - g0)) for g0 in range(0, groups, 4)]
+    else:
+        per = 4 // groups
+        for q0, ql in zip(batch.q_starts, batch.q_lens):
+            out += [(t, min(per, q0 + ql - t), 0, groups) for t in range(q0, q0 + ql, per)]
+    return np.asarray(out, dtype=np.int32).reshape(-1, 4)
+
+
 class TunedLatentAttention(PlainLatentAttention):
     def signature(self, batch, n_heads):
         return key_splits(batch, n_heads)
+
+    def metadata(self, batch, mixers):
+        """One list of blocks per number of head groups among the model's mixers."""
+        return {f"latent_tiles_{g}": shared_tiles(batch, g) for g in sorted({-(-m.n_heads // 16) for m in mixers})}
 
     def prepare(self, uk, uv, n_heads):
         w = LatentWeights(uk, uv, n_heads)
@@ -79,7 +104,11 @@ class TunedLatentAttention(PlainLatentAttention):
         else:
             ops.heads_matmul(q, w.uk, qa, H, transposed=False)
         z = rt.buffer("la_z", n, H * R, torch.float32)
-        if on_cores:
+        tiles = step.extra.get(f"latent_tiles_{-(-H // 16)}") if on_cores else None
+        if on_cores and tiles is not None and key_splits(step.host, H) == 1:
+            # a step of many rows (prompt portions): blocks of four waves share every chunk of keys through LDS
+            latent_attention_shared(qa, z, cache, step.positions, step.tok_seq, table, H, scale, window, tiles)
+        elif on_cores:
             n_split = key_splits(step.host, H)
             part_o = part_ml = None
             if n_split > 1:
@@ -125,6 +154,20 @@ def latent_attention_mfma(qa, z, cache, positions, tok_seq, block_table, n_heads
          ops._check(block_table, "latent_attention.block_table", torch.int32, (None, None)), block_table.shape[1],
          n, int(n_heads), R, cache.page_size, cache.n_pages, float(scale), int(window), int(n_split),
          part_o.data_ptr() if n_split > 1 else None, part_ml.data_ptr() if n_split > 1 else None, ops.stream_handle())
+    return z
+
+
+def latent_attention_shared(qa, z, cache, positions, tok_seq, block_table, n_heads, scale, window, tiles):
+    """The matrix-core kernel whose blocks share their keys; ``tiles``: ``shared_tiles`` on the device."""
+    n, R = qa.shape[0], cache.width
+    call("fl_latent_attention_shared", ops._check(qa, "latent_attention.qa", torch.bfloat16, (n, n_heads * R)),
+         ops._check(z, "latent_attention.z", torch.float32, (n, n_heads * R)),
+         ops._check(cache.pool, "latent_attention.pool", torch.bfloat16),
+         ops._check(positions, "latent_attention.positions", torch.int32, (n,)),
+         ops._check(tok_seq, "latent_attention.tok_seq", torch.int32, (n,)),
+         ops._check(block_table, "latent_attention.block_table", torch.int32, (None, None)), block_table.shape[1],
+         int(n_heads), R, cache.page_size, cache.n_pages, float(scale), int(window),
+         ops._check(tiles, "latent_attention.tiles", torch.int32, (None, 4)), tiles.shape[0], ops.stream_handle())
     return z
 
 

@@ -45,6 +45,11 @@ class LatentAttention(Mixer):
         """Into how many parts the kernels deal the keys: all that this mixer decides from the contexts' lengths."""
         return self.kernels.signature(batch, self.n_heads)
 
+    @classmethod
+    def step_metadata_for(cls, batch, mixers):
+        """The work lists the kernels of the mixers' runtime want for the batch."""
+        return mixers[0].kernels.metadata(batch, mixers) if mixers else {}
+
     def tensors(self):
         W, H, D, Dv, Rq, R = self.hidden_size, self.n_heads, self.head_dim, self.value_dim, self.q_rank, self.kv_rank
         t = {"dq.weight": TensorSpec((Rq, W)), "dq_norm.weight": TensorSpec((Rq,), "vector32"),

@@ -419,3 +419,38 @@ def test_keys_dealt_out_to_several_waves(splits):
     from flambeau_amd.kernels import ops
     ops.latent_attention(qa.float(), plain, cache, step.positions, step.tok_seq, step.block_tables[0], H, 0.5)
     assert (one - plain).abs().max().item() < 2e-2 * plain.abs().max().item()
+
+
+@pytest.mark.parametrize("H,R,ps", [(20, 96, 16), (32, 64, 32), (7, 512, 16), (40, 32, 16), (70, 160, 64)])
+def test_blocks_that_share_their_keys(H, R, ps):
+    """The matrix-core kernel whose four waves read every chunk of keys from LDS against the one whose waves
+    fetch for themselves: portions of unequal requests (some start mid-context, one is a single token, one
+    crosses several chunks), with one, two, three and more groups of 16 heads."""
+    from flambeau_amd.cache.storage import CacheStorage
+    from flambeau_amd.kernels import latent_attention as la
+    from flambeau_amd.parts import PagedRowSpec
+    n_pages = 64
+    store = CacheStorage([PagedRowSpec(R)], [None], torch.device(DEV), torch.bfloat16, n_pages=n_pages, page_size=ps, max_slots=4)
+    pool = store.pools[0]
+    pool[:, :, 0].normal_(0.0, 1.0)
+    pool[:, :, 1] = pool[:, :, 0].transpose(-1, -2).reshape(pool[:, :, 1].shape)
+    seqs = [(0, 150), (300, 7), (63, 1), (120, 70)]
+    step = make_step(seqs, ps, n_pages)
+    n = step.n_tokens
+    qa = (torch.randn(n, H * R, generator=torch.Generator().manual_seed(2)) * 0.4).to(torch.bfloat16).to(DEV)
+    cache = store.entries[0].kv
+    # rows beyond each request's newest token are poisoned: the kernels may load them but must not use them
+    for s, (st, q) in enumerate(seqs):
+        last = st + q
+        page = int(step.block_tables[0][s, last // ps]) if last % ps else -1
+        if page >= 0:
+            pool[0, page, 0, last % ps:] = float("nan")
+            pool[0, page, 1].view(R, ps)[:, last % ps:] = float("nan")
+    alone = torch.empty(n, H * R, dtype=torch.float32, device=DEV)
+    la.latent_attention_mfma(qa, alone, cache, step.positions, step.tok_seq, step.block_tables[0], H, 0.3)
+    tiles = torch.tensor(la.shared_tiles(step.host, -(-H // 16)), dtype=torch.int32, device=DEV)
+    shared = torch.full_like(alone, float("nan"))
+    la.latent_attention_shared(qa, shared, cache, step.positions, step.tok_seq, step.block_tables[0], H, 0.3, 0, tiles)
+    assert torch.isfinite(alone).all() and torch.isfinite(shared).all()
+    # (the two kernels round their weights against different bases: the shared one follows the maximum lazily)
+    assert (shared - alone).abs().max().item() < 5e-3 * alone.abs().max().item()
