@@ -96,7 +96,7 @@ int fl_heads_matmul_mfma_takes(int K, int J);
 // ---- the mLSTM recurrence (mlstm.hip) ----
 int fl_mlstm_scan(const float* proj, int ld, int col_q, int col_k, int col_v, int col_i, int col_f,
                   const float* bias_i, const float* bias_f, float cap, float q_scale, float* state,
-                  const int* seq_q_start, const int* seq_q_len, const int* seq_slots, float* out,
+                  const int* seq_q_start, const int* seq_q_len, const int* seq_slots, float* out, float* factors,
                   int n_seqs, int H, int D, int Dv, hipStream_t stream);
 int fl_mlstm_max_dim(void);
 long fl_mlstm_state_floats(int D, int Dv);

@@ -7,6 +7,8 @@
 //     m' = max(f + m, i);  a = exp(f + m - m');  b = exp(i - m')
 //     S <- a S + b k v^T;  n <- a n + b k;  m <- m'
 //     o = S^T q / (max(|n . q|, exp(-m)) + 1e-6)
+// Two kernels: the gates and their running maximum for all tokens (only the maximum is a chain there), then the
+// memory's walk with the factors exp(f + m - m'), exp(i - m'), exp(-m') ready.
 // The walk is the recurrence itself, so a prompt cut anywhere leaves the same state and the same o.
 #include "common.h"
 #include "api.h"
@@ -16,29 +18,80 @@
 #define ML_COLS 16           // columns of S per block
 #define ML_MAX_ROWS 32       // rows per thread: D <= ML_GROUP * ML_MAX_ROWS
 
+// v of the lane `n` places further round its row of 16 lanes (a data-parallel move between neighbouring lanes:
+// no trip through LDS, which is what a shuffle costs)
+template <int N>
+__device__ __forceinline__ float row_rotated(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + N, 0xf, 0xf, false));
+}
+// the sum over the 16 lanes of a row, in every lane
+__device__ __forceinline__ float row_sum16(float v) {
+    v += row_rotated<8>(v);
+    v += row_rotated<4>(v);
+    v += row_rotated<2>(v);
+    v += row_rotated<1>(v);
+    return v;
+}
+
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-// proj: float rows ld wide holding, per token, q [H][D] at col_q, k [H][D] at col_k, v [H][Dv] at col_v and
-// the gate pre-activations zi [H] at col_i, zf [H] at col_f.
+// The gates first, for all tokens of the step (fl_mlstm_scan's first kernel): per (request, head) a wave takes 64
+// tokens at a time, forms i and f in parallel, walks the running maximum m through them (a max-plus chain,
+// which is all that is sequential in the gates) and leaves for every token the three factors the memory's
+// walk needs: a = exp(f + m' - m), b = exp(i - m), c = exp(-m) (m' the maximum before the token).  The
+// head's m lives in the state behind S (the first float after it) and is read and written here alone.
+__global__ __launch_bounds__(64) void mlstm_gates_kernel(const float* __restrict__ proj, int ld, int col_i, int col_f,
+                                                         const float* __restrict__ bias_i, const float* __restrict__ bias_f, float cap,
+                                                         float* __restrict__ state, size_t rec, size_t m_at,
+                                                         const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
+                                                         const int* __restrict__ seq_slots, float* __restrict__ factors, int H) {
+    const int head = blockIdx.x, s = blockIdx.y, lane = threadIdx.x;
+    const int start = seq_q_start[s], len = seq_q_len[s];
+    float* mp = state + ((size_t)seq_slots[s] * H + head) * rec + m_at;
+    float m = *mp;
+    const float bi = bias_i ? bias_i[head] : 0.f, bf = bias_f ? bias_f[head] : 0.f;
+    for (int t0 = 0; t0 < len; t0 += 64) {
+        const int t = t0 + lane;
+        const bool live = t < len;
+        const float* row = proj + (size_t)(start + (live ? t : 0)) * ld;
+        const float gi = cap * tanhf((row[col_i + head] + bi) / cap);
+        const float gf = log_sigmoid(cap * tanhf((row[col_f + head] + bf) / cap));
+        float m_before = m, m_mine = m;
+        const int cnt = min(64, len - t0);
+        for (int u = 0; u < cnt; ++u) {                            // every lane walks the same chain and keeps its own link
+            const float mb = m;
+            m = fmaxf(__shfl(gf, u, FL_WAVE) + m, __shfl(gi, u, FL_WAVE));
+            if (u == lane) { m_before = mb; m_mine = m; }
+        }
+        if (live) {
+            float* f3 = factors + ((size_t)(start + t) * H + head) * 3;
+            f3[0] = expf(gf + m_before - m_mine);
+            f3[1] = expf(gi - m_mine);
+            f3[2] = expf(-m_mine);
+        }
+    }
+    if (lane == 0) *mp = m;
+}
+
+// proj: float rows ld wide holding, per token, q [H][D] at col_q, k [H][D] at col_k, v [H][Dv] at col_v;
+// factors [n][H][3] = (a, b, c) of mlstm_gates_kernel.
 // Block = (columns j0 .. j0 + 15, head, request); thread (g, c) holds S[d][j0 + c] for its rows d.
-// Every block walks n and m for itself and keeps a copy of its own in the state, since blocks of one
-// head start and end at different times: state [slots][H][D * Dv + blocks * (D + 1)], S first (column by
-// column, S[d][j] at j * D + d, so that the threads of a column read neighbours), then per block of
-// columns n [D] and m (fl_mlstm_state_floats gives the record's size).  A token's inputs are fetched
-// while the token before it is worked on.
+// Every block walks n for itself and keeps a copy of its own in the state, since blocks of one head start
+// and end at different times: state [slots][H][D * Dv + 1 + blocks * D], S first (column by column,
+// S[d][j] at j * D + d, so that the threads of a column read neighbours), then m, then per block of
+// columns n [D] (fl_mlstm_state_floats gives the record's size).
 template <int RPT>
 __global__ __launch_bounds__(ML_GROUP * ML_COLS) void mlstm_scan_kernel(
-    const float* __restrict__ proj, int ld, int col_q, int col_k, int col_v, int col_i, int col_f,
-    const float* __restrict__ bias_i, const float* __restrict__ bias_f, float cap, float q_scale,
+    const float* __restrict__ proj, int ld, int col_q, int col_k, int col_v, const float* __restrict__ factors, float q_scale,
     float* __restrict__ state, const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
-    const int* __restrict__ seq_slots, float* __restrict__ out, int H, int D, int Dv) {
+    const int* __restrict__ seq_slots, float* __restrict__ out, int H, int D, int Dv, int run) {
     const int g = threadIdx.x & (ML_GROUP - 1), c = threadIdx.x / ML_GROUP;
     const int j = blockIdx.x * ML_COLS + c, head = blockIdx.y, s = blockIdx.z;
     const bool live = j < Dv;
     const int start = seq_q_start[s], len = seq_q_len[s];
-    const size_t rec = (size_t)D * Dv + (size_t)gridDim.x * (D + 1);
+    const size_t rec = (size_t)D * Dv + 1 + (size_t)gridDim.x * D;
     float* st = state + ((size_t)seq_slots[s] * H + head) * rec;
-    float* mine = st + (size_t)D * Dv + (size_t)blockIdx.x * (D + 1);       // this block's n [D] and m
+    float* mine = st + (size_t)D * Dv + 1 + (size_t)blockIdx.x * D;         // this block's n [D]
     float S[RPT], nn[RPT];
 #pragma unroll
     for (int u = 0; u < RPT; ++u) {
@@ -46,50 +99,47 @@ __global__ __launch_bounds__(ML_GROUP * ML_COLS) void mlstm_scan_kernel(
         S[u] = (live && d < D) ? st[(size_t)j * D + d] : 0.f;
         nn[u] = d < D ? mine[d] : 0.f;
     }
-    float m = mine[D];
-    const float bi = bias_i ? bias_i[head] : 0.f, bf = bias_f ? bias_f[head] : 0.f;
-    float q[RPT], k[RPT], v = 0.f, zi = 0.f, zf = 0.f;
-    auto fetch = [&](int t, float* qn, float* kn, float& vn, float& zin, float& zfn) {
-        const float* row = proj + (size_t)(start + t) * ld;
-#pragma unroll
-        for (int u = 0; u < RPT; ++u) {
-            const int d = g + ML_GROUP * u;
-            qn[u] = d < D ? row[col_q + head * D + d] : 0.f;
-            kn[u] = d < D ? row[col_k + head * D + d] : 0.f;
+    // The step's tokens come through LDS a run at a time (q and k of the head, the block's 16 values, the three
+    // factors): one trip to memory per run instead of one per token, which is what the walk would wait for.
+    extern __shared__ float ml_smem[];
+    float* qs = ml_smem;                          // [run][D], scaled
+    float* ks = qs + (size_t)run * D;             // [run][D]
+    float* vs = ks + (size_t)run * D;             // [run][16]
+    float* fs = vs + (size_t)run * ML_COLS;       // [run][3]
+    for (int t0 = 0; t0 < len; t0 += run) {
+        const int cnt = min(run, len - t0);
+        __syncthreads();
+        for (int e = threadIdx.x; e < cnt * D; e += ML_GROUP * ML_COLS) {
+            const int tt = e / D, d = e - tt * D;
+            const float* row = proj + (size_t)(start + t0 + tt) * ld;
+            qs[e] = row[col_q + head * D + d] * q_scale;
+            ks[e] = row[col_k + head * D + d];
         }
-        vn = live ? row[col_v + head * Dv + j] : 0.f;
-        zin = row[col_i + head];
-        zfn = row[col_f + head];
-    };
-    if (len > 0) fetch(0, q, k, v, zi, zf);
-    for (int t = 0; t < len; ++t) {
-        float qn[RPT], kn[RPT], vn = 0.f, zin = 0.f, zfn = 0.f;
-        if (t + 1 < len) fetch(t + 1, qn, kn, vn, zin, zfn);
-#pragma unroll
-        for (int u = 0; u < RPT; ++u) q[u] *= q_scale;
-        const float gi = cap * tanhf((zi + bi) / cap);
-        const float gf = log_sigmoid(cap * tanhf((zf + bf) / cap));
-        const float m_new = fmaxf(gf + m, gi);
-        const float a = expf(gf + m - m_new), b = expf(gi - m_new);
-        m = m_new;
-        float num = 0.f, den = 0.f;
-#pragma unroll
-        for (int u = 0; u < RPT; ++u) {
-            S[u] = a * S[u] + b * k[u] * v;
-            nn[u] = a * nn[u] + b * k[u];
-            num = fmaf(S[u], q[u], num);
-            den = fmaf(nn[u], q[u], den);
+        for (int e = threadIdx.x; e < cnt * ML_COLS; e += ML_GROUP * ML_COLS) {
+            const int tt = e / ML_COLS, jj = blockIdx.x * ML_COLS + (e - tt * ML_COLS);
+            vs[e] = jj < Dv ? proj[(size_t)(start + t0 + tt) * ld + col_v + head * Dv + jj] : 0.f;
         }
-#pragma unroll
-        for (int off = ML_GROUP / 2; off > 0; off >>= 1) {
-            num += __shfl_xor(num, off, FL_WAVE);
-            den += __shfl_xor(den, off, FL_WAVE);
+        for (int e = threadIdx.x; e < cnt * 3; e += ML_GROUP * ML_COLS) {
+            const int tt = e / 3;
+            fs[e] = factors[((size_t)(start + t0 + tt) * H + head) * 3 + (e - tt * 3)];
         }
-        if (live && g == 0) out[((size_t)(start + t) * H + head) * Dv + j] = num / (fmaxf(fabsf(den), expf(-m)) + 1e-6f);
-        if (t + 1 < len) {
+        __syncthreads();
+        for (int tt = 0; tt < cnt; ++tt) {
+            const float fa = fs[3 * tt], fb = fs[3 * tt + 1], fc = fs[3 * tt + 2];
+            const float bv = fb * vs[tt * ML_COLS + c];
+            float num = 0.f, den = 0.f;
 #pragma unroll
-            for (int u = 0; u < RPT; ++u) { q[u] = qn[u]; k[u] = kn[u]; }
-            v = vn; zi = zin; zf = zfn;
+            for (int u = 0; u < RPT; ++u) {
+                const int d = g + ML_GROUP * u;
+                const float qv = d < D ? qs[tt * D + d] : 0.f, kv = d < D ? ks[tt * D + d] : 0.f;
+                S[u] = fa * S[u] + bv * kv;
+                nn[u] = fa * nn[u] + fb * kv;
+                num = fmaf(S[u], qv, num);
+                den = fmaf(nn[u], qv, den);
+            }
+            num = row_sum16(num);                                  // the 16 threads of a column are a row of lanes
+            den = row_sum16(den);
+            if (live && g == 0) out[((size_t)(start + t0 + tt) * H + head) * Dv + j] = num / (fmaxf(fabsf(den), fc) + 1e-6f);
         }
     }
 #pragma unroll
@@ -98,16 +148,15 @@ __global__ __launch_bounds__(ML_GROUP * ML_COLS) void mlstm_scan_kernel(
         if (live && d < D) st[(size_t)j * D + d] = S[u];
         if (c == 0 && d < D) mine[d] = nn[u];
     }
-    if (threadIdx.x == 0) mine[D] = m;
 }
 
 extern "C" int fl_mlstm_max_dim(void) { return ML_GROUP * ML_MAX_ROWS; }
 // floats of one head's record in the state
-extern "C" long fl_mlstm_state_floats(int D, int Dv) { return (long)D * Dv + (long)ceil_div(Dv, ML_COLS) * (D + 1); }
+extern "C" long fl_mlstm_state_floats(int D, int Dv) { return (long)D * Dv + 1 + (long)ceil_div(Dv, ML_COLS) * D; }
 
 extern "C" int fl_mlstm_scan(const float* proj, int ld, int col_q, int col_k, int col_v, int col_i, int col_f,
                              const float* bias_i, const float* bias_f, float cap, float q_scale, float* state,
-                             const int* seq_q_start, const int* seq_q_len, const int* seq_slots, float* out,
+                             const int* seq_q_start, const int* seq_q_len, const int* seq_slots, float* out, float* factors,
                              int n_seqs, int H, int D, int Dv, hipStream_t stream) {
     FL_CHECK(n_seqs >= 0 && H > 0 && D > 0 && Dv > 0, "mlstm_scan: bad sizes");
     FL_CHECK(D <= ML_GROUP * ML_MAX_ROWS, "mlstm_scan: %d key dims per head, at most %d", D, ML_GROUP * ML_MAX_ROWS);
@@ -116,12 +165,20 @@ extern "C" int fl_mlstm_scan(const float* proj, int ld, int col_q, int col_k, in
              "mlstm_scan: columns beyond rows %d wide", ld);
     if (n_seqs == 0) return 0;
     FL_CHECK(n_seqs <= 65535 && H <= 65535, "mlstm_scan: %d requests of %d heads are more than one grid takes", n_seqs, H);
+    FL_CHECK(factors, "mlstm_scan: no room for the gates' factors ([tokens][heads][3] floats)");
+    dim3 ggrid(H, n_seqs);
+    mlstm_gates_kernel<<<ggrid, 64, 0, stream>>>(proj, ld, col_i, col_f, bias_i, bias_f, cap, state, (size_t)fl_mlstm_state_floats(D, Dv),
+                                                 (size_t)D * Dv, seq_q_start, seq_q_len, seq_slots, factors, H);
+    FL_LAUNCH_CHECK();
     dim3 grid(ceil_div(Dv, ML_COLS), H, n_seqs);
     const int rpt = ceil_div(D, ML_GROUP);
+    // tokens per run through LDS: up to 32, as many as 60 KB hold
+    int run = (60 * 1024) / ((2 * D + ML_COLS + 3) * (int)sizeof(float));
+    run = run > 32 ? 32 : (run < 1 ? 1 : run);
+    const size_t lds = (size_t)run * (2 * D + ML_COLS + 3) * sizeof(float);
 #define FL_ML(R)                                                                                                      \
-    mlstm_scan_kernel<R><<<grid, ML_GROUP * ML_COLS, 0, stream>>>(proj, ld, col_q, col_k, col_v, col_i, col_f, bias_i, \
-                                                                  bias_f, cap, q_scale, state, seq_q_start, seq_q_len, \
-                                                                  seq_slots, out, H, D, Dv)
+    mlstm_scan_kernel<R><<<grid, ML_GROUP * ML_COLS, lds, stream>>>(proj, ld, col_q, col_k, col_v, factors, q_scale, state, \
+                                                                    seq_q_start, seq_q_len, seq_slots, out, H, D, Dv, run)
     if (rpt <= 1) FL_ML(1);
     else if (rpt <= 2) FL_ML(2);
     else if (rpt <= 4) FL_ML(4);

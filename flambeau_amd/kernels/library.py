@@ -39,7 +39,7 @@ _SIGNATURES = {
     "fl_latent_attention_mfma": [P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P],
     "fl_latent_attention_shared": [P, P, P, P, P, P, I, I, I, I, I, F, I, P, I, P],
     "fl_heads_matmul_mfma": [P, I, I, P, P, I, I, I, I, I, P, I, I, P],
-    "fl_mlstm_scan": [P, I, I, I, I, I, I, P, P, F, F, P, P, P, P, P, I, I, I, I, P],
+    "fl_mlstm_scan": [P, I, I, I, I, I, I, P, P, F, F, P, P, P, P, P, P, I, I, I, I, P],
     "fl_headnorm_gate": [P, P, P, I, I, P, I, I, I, I, F, P],
     "fl_moe_route": [P, I, I, I, I, I, I, I, P, P, P, P, P, I, P],
     "fl_moe_gemm": [P, I, P, P, P, P, P, I, I, I, P],

@@ -374,10 +374,11 @@ def mlstm_state_floats(dim: int, vdim: int) -> int:
     return int(lib.fl_mlstm_state_floats(int(dim), int(vdim)))
 
 
-def mlstm_scan(proj, cols, bias_i, bias_f, cap, q_scale, state, seq_q_start, seq_q_len, seq_slots, out, n_heads, dim, vdim):
+def mlstm_scan(proj, cols, bias_i, bias_f, cap, q_scale, state, seq_q_start, seq_q_len, seq_slots, out, factors, n_heads, dim, vdim):
     """The recurrence over the step's tokens, request by request, from and into ``state``
     ``[slots, heads, mlstm_state_floats]``.  ``proj``: float32 rows with q, k, v and the two gates'
-    pre-activations at the columns ``cols = (q, k, v, i, f)``; ``out`` float32 ``[n, heads * vdim]``."""
+    pre-activations at the columns ``cols = (q, k, v, i, f)``; ``out`` float32 ``[n, heads * vdim]``; ``factors``
+    float32 ``[n, heads * 3]``: room for the three factors per token and head that the gates' kernel leaves."""
     n, ld = proj.shape
     S = seq_q_start.shape[0]
     rec = mlstm_state_floats(dim, vdim)
@@ -389,7 +390,8 @@ def mlstm_scan(proj, cols, bias_i, bias_f, cap, q_scale, state, seq_q_start, seq
          float(cap), float(q_scale), _check(state, "mlstm_scan.state", torch.float32),
          _check(seq_q_start, "mlstm_scan.seq_q_start", torch.int32, (S,)), _check(seq_q_len, "mlstm_scan.seq_q_len", torch.int32, (S,)),
          _check(seq_slots, "mlstm_scan.seq_slots", torch.int32, (S,)),
-         _check(out, "mlstm_scan.out", torch.float32, (n, n_heads * vdim)), S, int(n_heads), int(dim), int(vdim), stream_handle())
+         _check(out, "mlstm_scan.out", torch.float32, (n, n_heads * vdim)),
+         _check(factors, "mlstm_scan.factors", torch.float32, (n, n_heads * 3)), S, int(n_heads), int(dim), int(vdim), stream_handle())
     return out
 
 

@@ -63,8 +63,9 @@ class MLstm(Mixer):
         proj = rt.buffer("ml_proj", n, self.w_in.rows, torch.float32)
         rt.gemm(x, self.w_in, proj)
         hidden = rt.buffer("ml_hidden", n, H * Dv, torch.float32)
+        factors = rt.buffer("ml_factors", n, 3 * H, torch.float32)
         ops.mlstm_scan(proj, self.cols, self.bias_i, self.bias_f, self.gate_cap, D ** -0.5, cache.state,
-                       step.seq_q_start, step.seq_q_len, step.seq_slots, hidden, H, D, Dv)
+                       step.seq_q_start, step.seq_q_len, step.seq_slots, hidden, factors, H, D, Dv)
         out = rt.buffer("ml_out", n, H * Dv)
         ops.headnorm_gate(hidden, self.norm, proj, self.gate_col, out, H, self.eps)
         return Product(out, self.w_o)
