@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_replay_in_all_cuttings(model_dirs, tmp_path, name, dtype):
     """The cache starts full of NaN, so a read of a row that was never written shows; the mixed trace
-    holds so many requests that the pool (sized, as the program's contract says, for the most
+    holds so many requests that the pool (sized, as the program's help says, for the most
     tokens live at a time, each request rounded up to 64) hands its pages out several times."""
     d = model_dirs[(name, dtype)]
     vocab = TINY[name]["config"]["vocab_size"]
