@@ -454,3 +454,38 @@ def test_blocks_that_share_their_keys(H, R, ps):
     assert torch.isfinite(alone).all() and torch.isfinite(shared).all()
     # (the two kernels round their weights against different bases: the shared one follows the maximum lazily)
     assert (shared - alone).abs().max().item() < 5e-3 * alone.abs().max().item()
+
+
+def test_the_command_line_serves_it(tmp_path):
+    """``random-weights`` -> ``inspect`` -> ``infer --json`` on a Kuvidra configuration, greedy in 32-bit with so
+    few slots and pages that requests wait and are pre-empted (a pre-empted request starts again from a
+    zeroed state): exactly the plain implementation's tokens."""
+    import json
+    import subprocess
+    import sys
+    cfg = CONFIGS["P"]["config"]
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    d = tmp_path / "model"
+
+    def cli(*args):
+        r = subprocess.run([sys.executable, "-m", "flambeau_amd", *map(str, args)], capture_output=True, text=True, timeout=600, cwd=str(rh.ROOT))
+        assert r.returncode == 0, f"{args}\n{r.stdout[-2000:]}\n{r.stderr[-4000:]}"
+        return r
+    cli("random-weights", "--config", tmp_path / "config.json", "--out", d, "--seed", 5, "--std", 0.16, "--gain-std", 0.1, "--dtype", "float32")
+    seen = cli("inspect", d).stdout
+    assert "architecture: Kuvidra" in seen and "tensors fit the model" in seen and "l1.mlp.shared.sg" in seen
+    prompts = list(rh.make_requests(97, [3, 30, 17], seed=6).values())
+    flags = []
+    for p in prompts:
+        flags += ["--prompt", ",".join(map(str, p))]
+    out = json.loads(cli("infer", "--model", d, *flags, "--max-tokens", 18, "--dtype", "float32", "--json", "--inflight-slots", 2,
+                         "--paged-kv", 5, "--page-size", 16, "--prefill-chunk-tokens", 16, "--max-queue-depth", 4).stdout)
+    conf, t = read_model(d)
+    for p, o in zip(prompts, out["outputs"]):
+        toks = list(p)
+        for tok in o:
+            logits = pk.forward(conf, t, toks)[-1]
+            best = int(np.argmax(logits))
+            assert tok == best or logits[best] - logits[tok] < 1e-4 * np.abs(logits).max()
+            toks.append(tok)
+        assert len(o) == 18
