@@ -88,6 +88,11 @@ int fl_latent_attention_shared(const void* qa, float* z, const void* pool, const
                                int page_size, int n_pages, float scale, int window, const int* tiles, int n_tiles,
                                hipStream_t stream);
 long fl_latent_attention_shared_lds(int R);
+// and for steps of few rows: a block of four waves per (token, 16 heads, part of the keys) that deal the latent's dims out among them
+int fl_latent_attention_dealt(const void* qa, float* z, const void* pool, const int* positions,
+                              const int* tok_seq, const int* block_table, int max_blocks, int n, int H, int R,
+                              int page_size, int n_pages, float scale, int window, int n_split, float* part_o,
+                              float* part_ml, hipStream_t stream);
 // out[t][h][j] = sum_k x[t][h][k] w[h][j][k] on the matrix cores (w bfloat16 [H][J][K])
 int fl_heads_matmul_mfma(const void* x, int x_dtype, int ldx, const void* w, void* out, int out_dtype, int n,
                          int H, int K, int J, const float* gate, int ldg, int gate_col0, hipStream_t stream);

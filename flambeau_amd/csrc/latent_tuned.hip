@@ -431,6 +431,192 @@ extern "C" int fl_latent_attention_shared(const void* qa, float* z, const void* 
 }
 FL_RECORDABLE(fl_latent_attention_shared)
 
+
+// The same walk for steps of few rows (decoding), where a wave that holds all of a latent's dims has no register
+// left for reads in flight and waits for every operand: the four waves of a block take one (token, 16 heads, part
+// of the keys) together and deal the latent's steps of 32 dims out among them (wave w: steps w, w + 4, ...).
+// Each forms its share of the scores, the shares are added through LDS in a fixed order (every wave gets the
+// same sums, hence the same maxima and weights), and each adds the weighted rows of its own dims.  A wave then
+// holds a quarter of the accumulators and queries, and the reads of a chunk are all in flight at once.
+template <int NSW>
+__global__ __launch_bounds__(64 * LT_WAVES) void latent_attention_dealt_kernel(
+    const bf16_t* __restrict__ qa, float* __restrict__ z, const bf16_t* __restrict__ pool,
+    const int* __restrict__ positions, const int* __restrict__ tok_seq, const int* __restrict__ block_table,
+    int max_blocks, int n, int H, int R, int page_size, int n_pages, float scale, int window, int groups_per_token,
+    int n_split, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    __shared__ f32x4 sx[LT_WAVES][4][64];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int unit = blockIdx.x;                                   // (token, group of 16 heads, part of the keys)
+    const int split = unit % n_split, tg = unit / n_split;
+    const int token = tg / groups_per_token, h0 = (tg - token * groups_per_token) * 16;
+    const int col = lane & 15, g = lane >> 4;
+    const int ns = R >> 5;
+    const int p = positions[token];
+    const int* table = block_table + (size_t)tok_seq[token] * max_blocks;
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const size_t page_stride = (size_t)2 * page_size * R;
+    const bool head_live = h0 + col < H;
+    bf16x8 qreg[NSW];
+    {
+        const bf16_t* qr = qa + ((size_t)token * H + h0 + (head_live ? col : 0)) * R;
+#pragma unroll
+        for (int i = 0; i < NSW; ++i) {
+            const int s = wave + LT_WAVES * i;
+            if (s < ns && head_live) {
+                const bf16x8 v = *(const bf16x8*)(qr + 32 * s + 8 * g);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qreg[i][e] = (bf16_t)((float)v[e] * scale);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qreg[i][e] = (bf16_t)0.f;
+            }
+        }
+    }
+    f32x4 o[2 * NSW];                                              // dims 32 s + 16 u + 4 g + r of the wave's steps s, u = 0, 1
+#pragma unroll
+    for (int t = 0; t < 2 * NSW; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    int first = lo & ~(LT_CHUNK - 1), last = p;
+    if (n_split > 1) {
+        const int chunks = (p - first) / LT_CHUNK + 1, per = (chunks + n_split - 1) / n_split;
+        last = min(p, first + (split + 1) * per * LT_CHUNK - 1);
+        first += split * per * LT_CHUNK;
+    }
+    for (int t0 = first; t0 <= last; t0 += LT_CHUNK) {
+        f32x4 sacc[4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            sacc[a] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            const int key = t0 + 32 * (a >> 1) + 8 * (col >> 2) + 4 * (a & 1) + (col & 3);
+            const int kc = min(key, p);
+            int page = table[kc / page_size];
+            page = min(max(page, 0), n_pages - 1);
+            const bf16_t* row = pool + (size_t)page * page_stride + (size_t)(kc % page_size) * R + 8 * g;
+#pragma unroll
+            for (int i = 0; i < NSW; ++i) {
+                const int s = wave + LT_WAVES * i;
+                if (s < ns) sacc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(row + 32 * s), qreg[i], sacc[a], 0, 0, 0);
+            }
+            sx[wave][a][lane] = sacc[a];
+        }
+        __syncthreads();
+        float cmax = -INFINITY;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            sacc[a] = (sx[0][a][lane] + sx[1][a][lane]) + (sx[2][a][lane] + sx[3][a][lane]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int key = t0 + 32 * (a >> 1) + 8 * g + 4 * (a & 1) + e;
+                if (key > p || key < lo) sacc[a][e] = -INFINITY;
+                cmax = fmaxf(cmax, sacc[a][e]);
+            }
+        }
+        __syncthreads();                                           // (the next chunk's shares overwrite sx)
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 16, FL_WAVE));
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 32, FL_WAVE));
+        const float m_new = fmaxf(m, cmax);
+        const float corr = expf(m - m_new);
+        m = m_new;
+        bf16x8 pb[2];
+        float lsum = 0.f;
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const bf16_t w = (bf16_t)expf(sacc[a][e] - m_new);
+                pb[a >> 1][4 * (a & 1) + e] = w;
+                lsum += (float)w;
+            }
+        lsum += __shfl_xor(lsum, 16, FL_WAVE);
+        lsum += __shfl_xor(lsum, 32, FL_WAVE);
+        l = l * corr + lsum;
+        const bool edge = t0 + LT_CHUNK - 1 > p || t0 < lo;
+        const bf16_t* cols[2];
+        int key0[2];
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            key0[q] = t0 + 32 * q + 8 * g;
+            const int kc = min(key0[q], p);
+            int page = table[kc / page_size];
+            page = min(max(page, 0), n_pages - 1);
+            cols[q] = pool + (size_t)page * page_stride + (size_t)page_size * R + (key0[q] % page_size);
+        }
+#pragma unroll
+        for (int t = 0; t < 2 * NSW; ++t) {
+            const int s = wave + LT_WAVES * (t >> 1);
+            if (s < ns) {
+                const int dim = 32 * s + 16 * (t & 1) + col;
+                o[t] *= corr;
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    bf16x8 v = *(const bf16x8*)(cols[q] + (size_t)dim * page_size);
+                    if (edge) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (key0[q] + e > p || key0[q] + e < lo) v[e] = (bf16_t)0.f;
+                    }
+                    o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pb[q], o[t], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (n_split > 1) {
+        float* po = part_o + ((size_t)unit * 16 + col) * R;
+#pragma unroll
+        for (int t = 0; t < 2 * NSW; ++t) {
+            const int s = wave + LT_WAVES * (t >> 1);
+            if (s < ns) *(f32x4*)(po + 32 * s + 16 * (t & 1) + 4 * g) = o[t];
+        }
+        if (wave == 0 && g == 0) {
+            part_ml[((size_t)unit * 16 + col) * 2] = m;
+            part_ml[((size_t)unit * 16 + col) * 2 + 1] = l;
+        }
+        return;
+    }
+    if (!head_live) return;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    float* zr = z + ((size_t)token * H + h0 + col) * R;
+#pragma unroll
+    for (int t = 0; t < 2 * NSW; ++t) {
+        const int s = wave + LT_WAVES * (t >> 1);
+        if (s < ns) *(f32x4*)(zr + 32 * s + 16 * (t & 1) + 4 * g) = o[t] * inv;
+    }
+}
+
+// fl_latent_attention_mfma with a block of four waves per (token, 16 heads, part of the keys): for steps of few rows
+extern "C" int fl_latent_attention_dealt(const void* qa, float* z, const void* pool, const int* positions,
+                                         const int* tok_seq, const int* block_table, int max_blocks, int n, int H, int R,
+                                         int page_size, int n_pages, float scale, int window, int n_split, float* part_o,
+                                         float* part_ml, hipStream_t stream) {
+    FL_CHECK(n >= 0 && H > 0 && n_pages > 0 && max_blocks > 0, "latent_attention_dealt: bad sizes");
+    FL_CHECK(n_split >= 1 && n_split <= 64 && (n_split == 1 || (part_o && part_ml)), "latent_attention_dealt: %d parts of the keys (at most 64) need a workspace", n_split);
+    FL_CHECK(fl_latent_attention_mfma_takes(R, page_size), "latent_attention_dealt: rows of %d values in pages of %d are not taken", R, page_size);
+    FL_CHECK((uintptr_t)qa % 16 == 0 && (uintptr_t)pool % 16 == 0 && (uintptr_t)z % 16 == 0, "latent_attention_dealt: operands must be 16-byte aligned");
+    FL_CHECK(window >= 0, "latent_attention_dealt: negative window");
+    if (n == 0) return 0;
+    const int groups = ceil_div(H, 16);
+    const long units = (long)n * groups * n_split;
+    FL_CHECK(units < (1L << 30), "latent_attention_dealt: too many rows");
+    const int nsw = ceil_div(R / 32, LT_WAVES);
+#define FL_LTD(NSW)                                                                                                       \
+    latent_attention_dealt_kernel<NSW><<<(unsigned)units, 64 * LT_WAVES, 0, stream>>>((const bf16_t*)qa, z, (const bf16_t*)pool, \
+                                                                                      positions, tok_seq, block_table, max_blocks, \
+                                                                                      n, H, R, page_size, n_pages, scale, window,  \
+                                                                                      groups, n_split, part_o, part_ml)
+    if (nsw <= 1) FL_LTD(1);
+    else if (nsw <= 2) FL_LTD(2);
+    else FL_LTD(4);
+#undef FL_LTD
+    FL_LAUNCH_CHECK();
+    if (n_split > 1) {
+        dim3 mgrid(n * H, ceil_div(R, 256));
+        latent_merge_kernel<<<mgrid, 256, 0, stream>>>(part_o, part_ml, z, H, R, groups, n_split);
+        FL_LAUNCH_CHECK();
+    }
+    return 0;
+}
+FL_RECORDABLE(fl_latent_attention_dealt)
+
 // ------------------------------------------------------------------ one product per head on the matrix cores
 // out[t][h][j] = sum_k x[t][h][k] w[h][j][k]   (x float or bfloat16 rows ldx apart, w bfloat16 [H][J][K], K a multiple
 // of 32, J of 16), optionally times sigmoid(gate[t][gate_col0 + h]).  A wave takes 16 tokens of one head: its x is

@@ -28,31 +28,60 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float* __restrict
     __shared__ int first[MOE_MAX_EXPERTS];
     for (int e = threadIdx.x; e < E; e += 1024) count[e] = 0;
     __syncthreads();
-    for (int t = threadIdx.x; t < n; t += 1024) {
+    // a wave per token: the lanes hold the token's logits (lane, lane + 64, ...), and every rank is a best-of-wave
+    // (the larger logit, the lower index among equals)
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int t = wave; t < n; t += 16) {
         const float* z = logits + (size_t)t * ld + col0;
+        float zv[MOE_MAX_EXPERTS / 64];
+#pragma unroll
+        for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) zv[u] = (lane + 64 * u < E) ? z[lane + 64 * u] : -INFINITY;
         float zmax = -INFINITY, zsum = 0.f;
         if (kind == 1) {
-            for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, z[e]);
-            for (int e = 0; e < E; ++e) zsum += expf(z[e] - zmax);
+#pragma unroll
+            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) zmax = fmaxf(zmax, zv[u]);
+            zmax = wave_max(zmax);
+#pragma unroll
+            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) zsum += (lane + 64 * u < E) ? expf(zv[u] - zmax) : 0.f;
+            zsum = wave_sum(zsum);
         }
         int chosen[MOE_MAX_TOP];
         float w[MOE_MAX_TOP], wsum = 0.f;
         for (int k = 0; k < top; ++k) {
-            int best = -1;
             float bz = -INFINITY;
-            for (int e = 0; e < E; ++e) {
-                bool taken = false;
-                for (int u = 0; u < k; ++u) taken |= chosen[u] == e;
-                if (!taken && (best < 0 || z[e] > bz)) { best = e; bz = z[e]; }
+            int best = 0x7fffffff;
+#pragma unroll
+            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+                const int e = lane + 64 * u;
+                if (e < E && (zv[u] > bz || (zv[u] == bz && e < best)) && zv[u] > -INFINITY) { bz = zv[u]; best = e; }
             }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const float oz = __shfl_xor(bz, off, FL_WAVE);
+                const int oe = __shfl_xor(best, off, FL_WAVE);
+                if (oz > bz || (oz == bz && oe < best)) { bz = oz; best = oe; }
+            }
+            if (best == 0x7fffffff) {                              // (only logits of minus infinity are left: the lowest index not yet taken)
+                best = 0;
+                for (int e = 0; e < E; ++e) {
+                    bool taken = false;
+                    for (int u = 0; u < k; ++u) taken |= chosen[u] == e;
+                    if (!taken) { best = e; break; }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u)
+                if (lane + 64 * u == best) zv[u] = -INFINITY;      // taken
             chosen[k] = best;
             w[k] = kind == 1 ? expf(bz - zmax) / zsum : 1.0f / (1.0f + expf(-bz));
             wsum += w[k];
         }
-        for (int k = 0; k < top; ++k) {
-            place[(size_t)t * top + k] = chosen[k];
-            pair_w[(size_t)t * top + k] = renorm ? w[k] / wsum : w[k];
-            atomicAdd(&count[chosen[k]], 1);
+        if (lane == 0) {
+            for (int k = 0; k < top; ++k) {
+                place[(size_t)t * top + k] = chosen[k];
+                pair_w[(size_t)t * top + k] = renorm ? w[k] / wsum : w[k];
+                atomicAdd(&count[chosen[k]], 1);
+            }
         }
     }
     __syncthreads();

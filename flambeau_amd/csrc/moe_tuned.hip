@@ -103,22 +103,21 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
     }
 }
 
-#define MT_STREAM_FEATURES 128       // output features per block of the streaming form: four waves of 32
-// The same for steps of few rows (decoding), where nearly every tile holds a row or two and all a block
-// does is stream its expert's weights: no LDS, no barrier.  out[p][:] = (scale[p] * x[src[p]]) W_e^T with
-// v_mfma_f32_16x16x32_bf16: a wave takes 32 features (two A operands, read straight from the expert's
-// rows) against up to four groups of 16 rows (B operands); K in steps of 32.  Row groups a tile does not
-// have are skipped, so a decode step (a row or two per expert) streams the weights once.
+#define MT_STREAM_FEATURES 32        // output features per block of the streaming form
+// The same for steps of few rows (decoding), where nearly every tile holds a row or two and all a block does is
+// stream its expert's weights: a block takes 32 features and its four waves deal the steps of K out among them
+// (wave w: steps w, w + 4, ...; together they read the rows end to end), so that even a step that touches four
+// experts has some hundred blocks; their sums are added through LDS in a fixed order.  No barrier inside the loop.
 __global__ __launch_bounds__(256) void moe_gemm_mfma_stream_kernel(const bf16_t* __restrict__ x, const int* __restrict__ src_row,
-                                                            const float* __restrict__ src_scale, const bf16_t* __restrict__ w,
-                                                            float* __restrict__ out, const int* __restrict__ tiles, int N, int K) {
+                                                                   const float* __restrict__ src_scale, const bf16_t* __restrict__ w,
+                                                                   float* __restrict__ out, const int* __restrict__ tiles, int N, int K) {
+    __shared__ f32x4 part[4][2][4][64];
     const int e = tiles[4 * blockIdx.y + 0];
     if (e < 0) return;
     const int p0 = tiles[4 * blockIdx.y + 1], M = tiles[4 * blockIdx.y + 2];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int col = lane & 15, g = lane >> 4;
-    const int f0 = blockIdx.x * MT_STREAM_FEATURES + wave * 32;
-    if (f0 >= N) return;
+    const int f0 = blockIdx.x * MT_STREAM_FEATURES;
     const bf16_t* we = w + (size_t)e * N * K;
     const bf16_t* wrow[2];
     bool wlive[2];
@@ -147,7 +146,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_stream_kernel(const bf16_t*
         for (int t = 0; t < 4; ++t) acc[a][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
     const bf16x8 zero = {(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
 #pragma unroll 4
-    for (int k0 = 0; k0 < K; k0 += 32) {
+    for (int k0 = 32 * wave; k0 < K; k0 += 128) {
         bf16x8 av[2], bv[4];
 #pragma unroll
         for (int a = 0; a < 2; ++a) av[a] = wlive[a] ? *(const bf16x8*)(wrow[a] + k0) : zero;
@@ -169,18 +168,26 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_stream_kernel(const bf16_t*
             }
     }
 #pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (t < groups) part[wave][a][t][lane] = acc[a][t];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
     for (int t = 0; t < 4; ++t) {
         if (!xlive[t] || t >= groups) continue;
         float* dst = out + (size_t)(p0 + 16 * t + col) * N;
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
+            const f32x4 sum = (part[0][a][t][lane] + part[1][a][t][lane]) + (part[2][a][t][lane] + part[3][a][t][lane]);
             const int f = f0 + 16 * a + 4 * g;
             if (f + 3 < N) {
-                *(f32x4*)(dst + f) = acc[a][t];
+                *(f32x4*)(dst + f) = sum;
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    if (f + r < N) dst[f + r] = acc[a][t][r];
+                    if (f + r < N) dst[f + r] = sum[r];
             }
         }
     }

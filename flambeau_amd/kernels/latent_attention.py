@@ -115,7 +115,8 @@ class TunedLatentAttention(PlainLatentAttention):
                 rows = n * -(-H // 16) * n_split * 16
                 part_o = rt.buffer("la_part_o", rows, R, torch.float32, max_rows=16 * (SPLIT_TARGET_WAVES + 64))
                 part_ml = rt.buffer("la_part_ml", rows, 2, torch.float32, max_rows=16 * (SPLIT_TARGET_WAVES + 64))
-            latent_attention_mfma(qa, z, cache, step.positions, step.tok_seq, table, H, scale, window, n_split, part_o, part_ml)
+            latent_attention_mfma(qa, z, cache, step.positions, step.tok_seq, table, H, scale, window, n_split, part_o, part_ml,
+                                  dealt=True)
         else:
             ops.latent_attention(qa, z, cache, step.positions, step.tok_seq, table, H, scale, window)
         if w.uv.dtype == torch.bfloat16 and lib.fl_heads_matmul_mfma_takes(R, Dv):
@@ -136,8 +137,9 @@ def heads_matmul_mfma(x, w, out, n_heads, gate=None, gate_col0=0):
 
 
 def latent_attention_mfma(qa, z, cache, positions, tok_seq, block_table, n_heads, scale, window=0, n_split=1,
-                          part_o=None, part_ml=None):
-    """``n_split`` > 1: every token's keys are dealt out to that many waves; ``part_o`` (float32, at least
+                          part_o=None, part_ml=None, dealt=False):
+    """``dealt``: the form with a block of four waves per (token, 16 heads, part of the keys), for steps of few rows
+    (else one wave each).  ``n_split`` > 1: every token's keys are dealt out to that many waves; ``part_o`` (float32, at least
     ``n * ceil(H / 16) * n_split * 16`` rows of R) and ``part_ml`` (as many rows of 2) hold their sums."""
     n, R = qa.shape[0], cache.width
     if n_split > 1:
@@ -146,7 +148,7 @@ def latent_attention_mfma(qa, z, cache, positions, tok_seq, block_table, n_heads
         ops._check(part_ml, "latent_attention.part_ml", torch.float32, (None, 2))
         if part_o.shape[0] < rows or part_ml.shape[0] < rows:
             raise ops.KernelError(f"latent_attention: {n_split} parts need {rows} rows of workspace")
-    call("fl_latent_attention_mfma", ops._check(qa, "latent_attention.qa", torch.bfloat16, (n, n_heads * R)),
+    call("fl_latent_attention_dealt" if dealt else "fl_latent_attention_mfma", ops._check(qa, "latent_attention.qa", torch.bfloat16, (n, n_heads * R)),
          ops._check(z, "latent_attention.z", torch.float32, (n, n_heads * R)),
          ops._check(cache.pool, "latent_attention.pool", torch.bfloat16),
          ops._check(positions, "latent_attention.positions", torch.int32, (n,)),

@@ -37,6 +37,7 @@ _SIGNATURES = {
     "fl_heads_matmul": [P, I, P, I, P, I, I, I, I, I, I, P, I, I, P],
     "fl_latent_attention": [P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
     "fl_latent_attention_mfma": [P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P],
+    "fl_latent_attention_dealt": [P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P],
     "fl_latent_attention_shared": [P, P, P, P, P, P, I, I, I, I, I, F, I, P, I, P],
     "fl_heads_matmul_mfma": [P, I, I, P, P, I, I, I, I, I, P, I, I, P],
     "fl_mlstm_scan": [P, I, I, I, I, I, I, P, P, F, F, P, P, P, P, P, P, I, I, I, I, P],

@@ -387,15 +387,16 @@ def test_trace_replay_as_a_program(dirs, tmp_path, dtype):
     close(got, ref, dtype, "trace_run")
 
 
+@pytest.mark.parametrize("H,R", [(20, 96), (5, 512), (33, 160), (16, 32)])
 @pytest.mark.parametrize("splits", [2, 8, 64])
-def test_keys_dealt_out_to_several_waves(splits):
+def test_keys_dealt_out_to_several_waves(splits, H, R):
     """The matrix-core attention kernel with every token's keys in several parts (what a decode step behind
     a long context does) against the same kernel in one part, rows of unequal contexts side by side, some
     shorter than the number of parts."""
     from flambeau_amd.cache.storage import CacheStorage
     from flambeau_amd.kernels import latent_attention as la
     from flambeau_amd.parts import PagedRowSpec
-    H, R, ps, n_pages = 20, 96, 16, 80
+    ps, n_pages = 16, 80
     store = CacheStorage([PagedRowSpec(R)], [None], torch.device(DEV), torch.bfloat16, n_pages=n_pages, page_size=ps, max_slots=4)
     pool = store.pools[0]                       # [entries, pages, 2, page, R]: rows, and the same rows transposed
     pool[:, :, 0].normal_(0.0, 1.0)
@@ -407,13 +408,18 @@ def test_keys_dealt_out_to_several_waves(splits):
     cache = store.entries[0].kv
     one = torch.empty(n, H * R, dtype=torch.float32, device=DEV)
     la.latent_attention_mfma(qa, one, cache, step.positions, step.tok_seq, step.block_tables[0], H, 0.5)
-    rows = n * 2 * splits * 16
+    rows = n * -(-H // 16) * splits * 16
     part_o = torch.full((rows, R), float("nan"), dtype=torch.float32, device=DEV)
     part_ml = torch.full((rows, 2), float("nan"), dtype=torch.float32, device=DEV)
     many = torch.empty_like(one)
     la.latent_attention_mfma(qa, many, cache, step.positions, step.tok_seq, step.block_tables[0], H, 0.5, 0, splits, part_o, part_ml)
     assert torch.isfinite(many).all()
     assert (many - one).abs().max().item() < 2e-3 * one.abs().max().item()
+    # the form in which four waves share a (token, 16 heads, part of the keys), in parts and whole
+    for k in (splits, 1):
+        dealt = torch.full_like(one, float("nan"))
+        la.latent_attention_mfma(qa, dealt, cache, step.positions, step.tok_seq, step.block_tables[0], H, 0.5, 0, k, part_o, part_ml, dealt=True)
+        assert torch.isfinite(dealt).all() and (dealt - one).abs().max().item() < 2e-3 * one.abs().max().item(), k
     # and both against the float kernel
     plain = torch.empty_like(one)
     from flambeau_amd.kernels import ops
