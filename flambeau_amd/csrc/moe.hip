@@ -1,7 +1,8 @@
 // A feed-forward of routed experts: the router's choice, the experts' products over the rows each
 // was given, and the sum per token.
 //
-//   fl_moe_route    scores -> for every token its `top` experts (largest router logits, the lower index among
+//   fl_moe_route    (two kernels: the picks, a wave per token; then one block that counts and sorts)
+//                   scores -> for every token its `top` experts (largest router logits, the lower index among
 //                   equals) and their weights; the (token, expert) pairs sorted by expert, cut into row
 //                   tiles that each belong to one expert
 //   fl_moe_gemm     out[p] = (scale[p] * x[src[p]]) W_e^T for the sorted pairs p, e the expert of p's tile
@@ -20,29 +21,25 @@
 // kind 1: weight = softmax over all experts.  renorm: the chosen weights are divided by their sum.
 // place [n * top]: where pair (t, k) lies in the sorted order; src_row / src_scale [n * top]: token and weight
 // of every sorted place; tiles [max_tiles][4] = (expert, first place, places, 0), expert -1: unused.
-__global__ __launch_bounds__(1024) void moe_route_kernel(const float* __restrict__ logits, int ld, int col0, int n, int E,
-                                                         int top, int kind, int renorm, int* __restrict__ place,
-                                                         int* __restrict__ src_row, float* __restrict__ src_scale,
-                                                         float* __restrict__ pair_w, int* __restrict__ tiles, int max_tiles) {
-    __shared__ int count[MOE_MAX_EXPERTS];
-    __shared__ int first[MOE_MAX_EXPERTS];
-    for (int e = threadIdx.x; e < E; e += 1024) count[e] = 0;
-    __syncthreads();
+__global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__ logits, int ld, int col0, int n, int E,
+                                                       int top, int kind, int renorm, int* __restrict__ place,
+                                                       float* __restrict__ pair_w) {
     // a wave per token: the lanes hold the token's logits (lane, lane + 64, ...), and every rank is a best-of-wave
     // (the larger logit, the lower index among equals)
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    for (int t = wave; t < n; t += 16) {
+    const int lane = threadIdx.x & 63;
+    const int nu = (E + 63) >> 6;
+    for (int t = blockIdx.x * 4 + (threadIdx.x >> 6); t < n; t += gridDim.x * 4) {
         const float* z = logits + (size_t)t * ld + col0;
         float zv[MOE_MAX_EXPERTS / 64];
 #pragma unroll
-        for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) zv[u] = (lane + 64 * u < E) ? z[lane + 64 * u] : -INFINITY;
+        for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) zv[u] = (u < nu && lane + 64 * u < E) ? z[lane + 64 * u] : -INFINITY;
         float zmax = -INFINITY, zsum = 0.f;
         if (kind == 1) {
 #pragma unroll
-            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) zmax = fmaxf(zmax, zv[u]);
+            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) if (u < nu) zmax = fmaxf(zmax, zv[u]);
             zmax = wave_max(zmax);
 #pragma unroll
-            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) zsum += (lane + 64 * u < E) ? expf(zv[u] - zmax) : 0.f;
+            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) zsum += (u < nu && lane + 64 * u < E) ? expf(zv[u] - zmax) : 0.f;
             zsum = wave_sum(zsum);
         }
         int chosen[MOE_MAX_TOP];
@@ -53,7 +50,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float* __restrict
 #pragma unroll
             for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
                 const int e = lane + 64 * u;
-                if (e < E && (zv[u] > bz || (zv[u] == bz && e < best)) && zv[u] > -INFINITY) { bz = zv[u]; best = e; }
+                if (u < nu && e < E && (zv[u] > bz || (zv[u] == bz && e < best)) && zv[u] > -INFINITY) { bz = zv[u]; best = e; }
             }
 #pragma unroll
             for (int off = 32; off > 0; off >>= 1) {
@@ -71,7 +68,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float* __restrict
             }
 #pragma unroll
             for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u)
-                if (lane + 64 * u == best) zv[u] = -INFINITY;      // taken
+                if (u < nu && lane + 64 * u == best) zv[u] = -INFINITY;      // taken
             chosen[k] = best;
             w[k] = kind == 1 ? expf(bz - zmax) / zsum : 1.0f / (1.0f + expf(-bz));
             wsum += w[k];
@@ -80,10 +77,20 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float* __restrict
             for (int k = 0; k < top; ++k) {
                 place[(size_t)t * top + k] = chosen[k];
                 pair_w[(size_t)t * top + k] = renorm ? w[k] / wsum : w[k];
-                atomicAdd(&count[chosen[k]], 1);
             }
         }
     }
+}
+
+// The (token, expert) pairs that moe_pick_kernel left (place[pair] = expert) counted, sorted by expert and cut into tiles.
+__global__ __launch_bounds__(1024) void moe_route_kernel(int n, int E, int top, int* __restrict__ place,
+                                                         int* __restrict__ src_row, float* __restrict__ src_scale,
+                                                         const float* __restrict__ pair_w, int* __restrict__ tiles, int max_tiles) {
+    __shared__ int count[MOE_MAX_EXPERTS];
+    __shared__ int first[MOE_MAX_EXPERTS];
+    for (int e = threadIdx.x; e < E; e += 1024) count[e] = 0;
+    __syncthreads();
+    for (int a = threadIdx.x; a < n * top; a += 1024) atomicAdd(&count[place[a]], 1);
     __syncthreads();
     if (threadIdx.x == 0) {
         int at = 0, tile = 0;
@@ -129,7 +136,10 @@ extern "C" int fl_moe_route(const float* logits, int ld, int col0, int n, int E,
     }
     FL_CHECK(kind == 0 || kind == 1, "moe_route: unknown scoring %d", kind);
     if (n == 0) return 0;
-    moe_route_kernel<<<1, 1024, 0, stream>>>(logits, ld, col0, n, E, top, kind, renorm, place, src_row, src_scale, pair_w, tiles, max_tiles);
+    const int pick_blocks = n < 4 * 1024 ? (n + 3) / 4 : 1024;
+    moe_pick_kernel<<<pick_blocks, 256, 0, stream>>>(logits, ld, col0, n, E, top, kind, renorm, place, pair_w);
+    FL_LAUNCH_CHECK();
+    moe_route_kernel<<<1, 1024, 0, stream>>>(n, E, top, place, src_row, src_scale, pair_w, tiles, max_tiles);
     FL_LAUNCH_CHECK();
     return 0;
 }
