@@ -132,3 +132,30 @@ def test_routed_experts_plain():
     one = pk.moe_ff(h, t, "f.", {"router": {"experts": E, "top": 1}})
     best = s.argmax(axis=1)
     assert np.allclose(one[2], pk.gated_expert(s[2, best[2]] * h[2:3], t, f"f.e{best[2]}.")[0])
+
+
+def test_work_lists_of_the_attention_kernels():
+    """The blocks of the kernel that shares its keys cover every (token, group of 16 heads) once, hold at most four
+    waves and never cross a request; the number of parts the keys are dealt into is a power of two that follows
+    the rows and the longest context."""
+    from flambeau_amd.kernels.latent_attention import key_splits, shared_tiles
+    from flambeau_amd.parts import HostBatch
+    batch = HostBatch([0, 7, 8, 21], [7, 1, 13, 2], [0, 99, 5, 0], [0, 1, 2, 3], 23, 0)
+    for groups in (1, 2, 3, 4, 5, 9):
+        tiles = shared_tiles(batch, groups)
+        seen = set()
+        for t0, nt, g0, ng in tiles.tolist():
+            assert 1 <= nt * ng <= 4
+            owner = [s for s, (q0, ql) in enumerate(zip(batch.q_starts, batch.q_lens)) if q0 <= t0 < q0 + ql]
+            assert len(owner) == 1 and t0 + nt <= batch.q_starts[owner[0]] + batch.q_lens[owner[0]]
+            for t in range(t0, t0 + nt):
+                for g in range(g0, g0 + ng):
+                    assert (t, g) not in seen
+                    seen.add((t, g))
+        assert seen == {(t, g) for t in range(23) for g in range(groups)}
+    one = HostBatch([0], [1], [4000], [0], 1, 0)
+    assert key_splits(one, 32) == 32 and key_splits(one, 8) == 32          # 4,001 keys: 62 chunks, the next power of two below
+    assert key_splits(HostBatch([0], [1], [100], [0], 1, 0), 8) == 1
+    assert key_splits(HostBatch([0], [2048], [0], [0], 2048, 0), 32) == 1
+    many = HostBatch(list(range(64)), [1] * 64, [3000] * 64, list(range(64)), 64, 0)
+    assert key_splits(many, 32) == 8
