@@ -129,6 +129,9 @@ def run_mixer(mixer, rt, x, cuts, page_size=8, n_pages=40):
     got, at = [], 0
     for k in cuts:
         step = make_step([(at, k)], page_size, n_pages, slots=[2], seed=1)
+        if hasattr(mixer, "step_metadata_for"):                # the work lists the step function would upload
+            step.extra.update({name: torch.tensor(arr, dtype=torch.int32, device=DEV)
+                               for name, arr in type(mixer).step_metadata_for(step.host, [mixer]).items()})
         r = mixer.forward(x[at:at + k].to(DEV).contiguous(), step, store.entries[0])
         r = r.compute(rt) if isinstance(r, Product) else r
         got.append(r.double().cpu().numpy())
@@ -495,3 +498,33 @@ def test_the_command_line_serves_it(tmp_path):
             assert tok == best or logits[best] - logits[tok] < 1e-4 * np.abs(logits).max()
             toks.append(tok)
         assert len(o) == 18
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("R,window", [(24, 13), (64, 70), (96, 64), (32, 1)])
+def test_latent_attention_with_a_window(dtype, R, window):
+    """``window`` keys, the query's own included (no model of the package sets it yet): the mixer against the
+    formula written out, whole and in portions that cross the window's edge and the kernels' chunks of 64 keys;
+    pages that the window has passed are poisoned as a manager that returns them would leave them."""
+    from flambeau_amd.parts import MIXERS, PartSpec
+    rt = make_rt(dtype)
+    W, n, eps, H, D, Dv, Rq = 40, 150, 1e-5, 5, 32, 16, 16
+    mixer, plain = bound_part(MIXERS, PartSpec("latent_attention", dict(hidden_size=W, n_heads=H, head_dim=D, value_dim=Dv, q_rank=Rq,
+                                                                         kv_rank=R, scale=0.2, eps=eps, window=window)), dtype, rt, seed=R)
+    assert mixer.cache_spec().window == window
+    x = (torch.randn(n, W, generator=torch.Generator().manual_seed(8))).to(TORCH[dtype])
+    h = x.double().numpy()
+    cq = pk.rms_norm(h @ plain["m.dq"].T, plain["m.dq.norm"], eps)
+    q = (cq @ plain["m.uq"].T).reshape(n, H, D)
+    c = pk.rms_norm(h @ plain["m.dkv"].T, plain["m.dkv.norm"], eps)
+    k, v = (c @ plain["m.uk"].T).reshape(n, H, D), (c @ plain["m.uv"].T).reshape(n, H, Dv)
+    want = np.zeros((n, H, Dv))
+    for i in range(n):
+        lo = max(0, i - window + 1)
+        s = np.einsum("hd,jhd->hj", q[i], k[lo:i + 1]) * 0.2
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        want[i] = np.einsum("hj,jhv->hv", p / p.sum(axis=1, keepdims=True), v[lo:i + 1])
+    want = (want * pk.sigmoid(h @ plain["m.g"].T)[:, :, None]).reshape(n, H * Dv) @ plain["m.o"].T
+    for cuts in ([n], [60, 5, 1, 1, 2, 30, 2, 6, 1, 42], [1] * 90 + [60]):
+        got = run_mixer(mixer, rt, x, cuts)
+        assert np.abs(got - want).max() < (3e-5 if dtype == "float32" else 3e-2) * np.abs(want).max(), cuts
