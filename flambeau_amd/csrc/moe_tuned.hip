@@ -8,7 +8,7 @@
 
 // out[p][:] = (scale[p] * x[src[p]]) W_e^T over the tiles of fl_moe_route, as fl_moe_gemm computes it, with
 // v_mfma_f32_16x16x32_bf16, K in steps of 32.  A wave takes 64 features (four A operands, read straight
-// from the expert's rows, a step ahead) against the tile's rows in groups of 16 (B operands).  The rows
+// from the expert's rows, four steps ahead) against the tile's rows in groups of 16 (B operands).  The rows
 // are gathered, scaled and rounded once per block and shared through LDS (two slots, one barrier a
 // step; the 16-byte pieces of a row are exchanged by (row / 2) % 4 so that the reads of a group of
 // rows meet in no bank).  Row groups a tile does not have are skipped, so a decode step (a row or two
@@ -54,35 +54,43 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
     for (int a = 0; a < 4; ++a)
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[a][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    bf16x8 av[4];
+    // The weights and the rows' pieces of a step are asked for four steps before they are used (a ring of registers):
+    // a trip to memory takes some thousand clocks, the products of a step a few hundred.
+    const int steps = K >> 5;
+    bf16x8 avq[4][4], xq[4];
 #pragma unroll
-    for (int a = 0; a < 4; ++a) av[a] = wlive[a] ? *(const bf16x8*)(wrow[a]) : zero;
-    xs[0][sslot] = staged(0);
+    for (int d = 0; d < 4; ++d) {
+        if (d < steps) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) avq[d][a] = wlive[a] ? *(const bf16x8*)(wrow[a] + 32 * d) : zero;
+            xq[d] = staged(32 * d);
+        }
+    }
+    xs[0][sslot] = xq[0];
     __syncthreads();
-    int cur = 0;
-    for (int k0 = 0; k0 < K; k0 += 32) {
-        const bool more = k0 + 32 < K;
-        bf16x8 an[4], xn = zero;
-        if (more) {
+    for (int s0 = 0; s0 < steps; s0 += 4) {
 #pragma unroll
-            for (int a = 0; a < 4; ++a) an[a] = wlive[a] ? *(const bf16x8*)(wrow[a] + k0 + 32) : zero;
-            xn = staged(k0 + 32);
-        }
+        for (int j = 0; j < 4; ++j) {
+            const int s_now = s0 + j;
+            if (s_now < steps) {                                   // (the same for every thread of the block)
+                const int cur = j & 1;
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
-            if (t < groups) {
-                const int r = 16 * t + col;
-                const bf16x8 bv = xs[cur][r * 4 + (g ^ ((r >> 1) & 3))];
+                for (int t = 0; t < 4; ++t)
+                    if (t < groups) {
+                        const int r = 16 * t + col;
+                        const bf16x8 bv = xs[cur][r * 4 + (g ^ ((r >> 1) & 3))];
 #pragma unroll
-                for (int a = 0; a < 4; ++a) acc[a][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[a], bv, acc[a][t], 0, 0, 0);
+                        for (int a = 0; a < 4; ++a) acc[a][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(avq[j][a], bv, acc[a][t], 0, 0, 0);
+                    }
+                if (s_now + 1 < steps) xs[cur ^ 1][sslot] = xq[(j + 1) & 3];
+                if (s_now + 4 < steps) {
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) avq[j][a] = wlive[a] ? *(const bf16x8*)(wrow[a] + 32 * (s_now + 4)) : zero;
+                    xq[j] = staged(32 * (s_now + 4));
+                }
+                __syncthreads();
             }
-        if (more) {
-            xs[cur ^ 1][sslot] = xn;
-#pragma unroll
-            for (int a = 0; a < 4; ++a) av[a] = an[a];
         }
-        __syncthreads();
-        cur ^= 1;
     }
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
