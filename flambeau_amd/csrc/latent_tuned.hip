@@ -646,6 +646,7 @@ __global__ __launch_bounds__(64 * LT_WAVES) void heads_matmul_mfma_kernel(
     }
     const float gv = (gate && live) ? 1.0f / (1.0f + expf(-gate[(size_t)token * ldg + gate_col0 + h])) : 1.0f;
     const bf16_t* wh = w + (size_t)h * J * K;
+#pragma unroll 4
     for (int jt = j_first; jt < J / 16; jt += j_parts) {
         f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
         const bf16_t* row = wh + (size_t)(16 * jt + col) * K + 8 * g;
