@@ -106,7 +106,7 @@ int fl_mlstm_scan(const float* proj, int ld, int col_q, int col_k, int col_v, in
 int fl_mlstm_max_dim(void);
 long fl_mlstm_state_floats(int D, int Dv);
 int fl_headnorm_gate(const float* x, const float* w, const float* gate, int ldg, int gate_col0, void* out,
-                     int out_dtype, int n, int H, int Dv, float eps, hipStream_t stream);
+                     int out_dtype, int n, int H, int Dv, float eps, int gate_kind, hipStream_t stream);
 
 // ---- routed experts, activations, re-entry of the stream (moe.hip) ----
 int fl_moe_route(const float* logits, int ld, int col0, int n, int E, int top, int kind, int renorm,
@@ -247,6 +247,60 @@ int fl_attn_prefill_splits(int n_tiles, int nh, int nkv, int hd, int max_keys);
 int fl_attn_prefill_heads(int n_tiles, int nh, int nkv, int hd, int max_keys);      // query heads per wave: the qt_hint to pass
 int fl_attn_prefill_workspace(int n_rows, int nh, int hd, int n_split, long* o_floats, long* ml_floats);
 int fl_attn_decode_workspace(int n_items, int nh, int hd, int n_split, long* o_floats, long* ml_floats);
+
+// ---- the same attention kernels with capped scores: score <- softcap * tanh(score / softcap) ----
+int fl_attn_plain_capped(const void* q, void* out, const void* cache_base, int dtype,
+                         const int* positions, const int* tok_seq, const int* block_table,
+                         int max_blocks, int n, int nh, int nkv, int hd, int page_size, int n_pages,
+                         float scale, int window, float softcap, hipStream_t stream);
+int fl_attn_decode_items_capped(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
+                                const int* items, int n_items, const int* block_table, int max_blocks, int nh,
+                                int nkv, int hd, int page_size, int n_pages, float scale, int window,
+                                float softcap, const int* firsts, int n_rows, hipStream_t stream);
+int fl_attn_prefill_capped(const void* q, void* out, const void* cache_base, const int* tiles,
+                           int n_tiles, const int* positions, const int* block_table,
+                           int max_blocks, int nh, int nkv, int hd, int page_size, int n_pages,
+                           float scale, int window, float softcap, int qt_hint, float* part_o, float* part_ml,
+                           int n_split, hipStream_t stream);
+
+// ---- rows of the residual stream and of mixers' outputs (stream_ops.hip) ----
+// out = tanh(alpha * (x + delta)) * w + b (Dynamic Tanh); resid_out, rows as for fl_rmsnorm
+int fl_dyt(const float* x, const float* delta, float* resid_out, const int* rows, const float* alpha,
+           const float* w, const float* b, void* out, int out_dtype, int n_rows, int H, hipStream_t stream);
+int fl_embed_scaled(const void* table, int dtype, const int* tokens, float* out, int n, int H, int V, float scale,
+                    hipStream_t stream);
+// out[r][i] = act(gu[r][i]) * gu[r][I + i]; kinds as fl_activation
+int fl_gated_act(const float* gu, void* out, int out_dtype, int n, int I, int kind, hipStream_t stream);
+// out = ca * a / rms(a) * wa + cb * b / rms(b) * wb per row
+int fl_norm_mix(const float* a, const float* wa, float ca, const float* b, const float* wb, float cb, float* out,
+                int n, int H, float eps, hipStream_t stream);
+// out[t][h][j < Dv] = x[t][h][j] * g(gate[t][gate_col0 + h * Dv + j]), heads of x ldh wide; g: 0 none, 1 sigmoid, 2 silu
+int fl_heads_gate(const void* x, int dtype, int ldh, const float* gate, int ldg, int gate_col0, int kind, void* out,
+                  int n, int H, int Dv, hipStream_t stream);
+
+// ---- between a joined q/k/v projection and attention (qkv_prepare.hip) ----
+int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, int col_v, const int* positions,
+                   const int* tok_seq, const int* block_table, int max_blocks, void* q_out, void* cache_base,
+                   int dtype, int n, int nh, int nkv, int D, int Dv, int hdp, int page_size, int n_pages, int rot,
+                   int interleaved, const float* cs, const float* qnorm_w, const float* knorm_w, int head_norm,
+                   float eps, float* v_first, int vmix_mode, const float* lambda, int write_cache,
+                   hipStream_t stream);
+
+// ---- linear recurrences with a matrix state per head (linear_scan.hip) ----
+int fl_linear_scan_max_dim(void);
+int fl_conv_max_taps(void);
+int fl_linear_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
+                   const float* head_decay, const float* tok_decay, const float* beta, int ldg, float* state,
+                   long slot_stride, const int* seq_q_start, const int* seq_q_len, const int* seq_slots,
+                   float* out, int n_seqs, int H, int G, int D, int Dv, hipStream_t stream);
+int fl_conv_prepare(const float* proj, int ld, int col0, int col_b, int col_a, const float* conv_w,
+                    const float* a_log, const float* dt_bias, float* conv_state, long slot_stride,
+                    const int* tok_seq, const int* seq_q_start, const int* seq_q_len, const int* seq_slots,
+                    float* prep, float* gates, int n, int n_seqs, int G, int H, int D, int Dv, int taps,
+                    float q_scale, float unit_eps, hipStream_t stream);
+int fl_rotate_scale(const float* proj, int ld, int col_a, int col_b, const float* cs, int rot, int interleaved,
+                    float scale_a, float scale_b, float* out_a, float* out_b, int n, int H, int D,
+                    hipStream_t stream);
 
 // ---- step programs (program.hip): launches recorded once, replayed with one call ----
 typedef union FlArg { void* p; long l; int i; float f; } FlArg;

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256, HDP <= 128 ? 2 : 1) void attn_decode_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* part_o,
     float* part_ml, PagedCache cache, const int4* __restrict__ items,
     const int* __restrict__ block_table, int max_blocks, int nh, float scale, int window,
-    int n_split, int q_tiles, int ps_shift, int item_base) {
+    int n_split, int q_tiles, int ps_shift, int item_base, float softcap) {
     constexpr int QS = HDP / 32;     // k-steps of the score product
     constexpr int DT = HDP / 16;     // 16-wide tiles of head dims in the output
     constexpr bool PIPELINED = HDP <= 128;       // two chunks of keys and values fit the registers
@@ -143,8 +143,13 @@ __global__ __launch_bounds__(256, HDP <= 128 ? 2 : 1) void attn_decode_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int ka = t0 + 8 * g + r, kb = ka + 4;
-            sa[r] = (ka >= lo && ka <= p) ? sa[r] * scale : -INFINITY;
-            sb[r] = (kb >= lo && kb <= p) ? sb[r] * scale : -INFINITY;
+            float va = sa[r] * scale, vb = sb[r] * scale;
+            if (softcap > 0.f) {                             // scores capped smoothly at +-softcap
+                va = softcap * tanhf(va / softcap);
+                vb = softcap * tanhf(vb / softcap);
+            }
+            sa[r] = (ka >= lo && ka <= p) ? va : -INFINITY;
+            sb[r] = (kb >= lo && kb <= p) ? vb : -INFINITY;
             mt = fmaxf(mt, fmaxf(sa[r], sb[r]));
         }
         mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
@@ -314,7 +319,7 @@ static int attn_decode_launch(const char* who, const void* q, void* out, float* 
                               const void* cache_base, const int* items, int n_items, const int* block_table,
                               int max_blocks, int nh, int nkv, int hd, int page_size, int n_pages,
                               float scale, int window, int n_split, hipStream_t stream, bool own_splits = false,
-                              const int* firsts = nullptr, int n_rows = 0) {
+                              const int* firsts = nullptr, int n_rows = 0, float softcap = 0.f) {
     FL_CHECK(n_items >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "%s: bad head counts %d/%d", who, nh, nkv);
     FL_CHECK(hd > 0 && hd <= 256 && hd % 8 == 0, "%s: head size %d must be a multiple of 8 up to 256", who, hd);
     FL_CHECK(page_size % 8 == 0, "%s: page size %d must be a multiple of 8", who, page_size);
@@ -336,7 +341,7 @@ static int attn_decode_launch(const char* who, const void* q, void* out, float* 
 #define FL_DEC(HDP_)                                                                                  \
     attn_decode_kernel<HDP_><<<grid, 256, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, part_o, part_ml, c,       \
                                                        (const int4*)items, block_table, max_blocks, nh, scale,   \
-                                                       window, n_split, q_tiles, ps_shift, item_base)
+                                                       window, n_split, q_tiles, ps_shift, item_base, softcap)
         switch (hdp) {
             case 32: FL_DEC(32); break;
             case 64: FL_DEC(64); break;
@@ -390,6 +395,18 @@ extern "C" int fl_attn_decode_items(const void* q, void* out, float* part_o, flo
                               nh, nkv, hd, page_size, n_pages, scale, window, 1, stream, true, firsts, n_rows);
 }
 FL_RECORDABLE(fl_attn_decode_items)
+
+// the same with the scores capped: score <- softcap * tanh(score / softcap) before the softmax (softcap > 0)
+extern "C" int fl_attn_decode_items_capped(const void* q, void* out, float* part_o, float* part_ml, const void* cache_base,
+                                           const int* items, int n_items, const int* block_table, int max_blocks, int nh,
+                                           int nkv, int hd, int page_size, int n_pages, float scale, int window,
+                                           float softcap, const int* firsts, int n_rows, hipStream_t stream) {
+    FL_CHECK(!firsts || (part_o && part_ml), "attn_decode_items: needs a workspace");
+    FL_CHECK(softcap >= 0.f, "attn_decode_items: negative cap");
+    return attn_decode_launch("attn_decode_items", q, out, part_o, part_ml, cache_base, items, n_items, block_table, max_blocks,
+                              nh, nkv, hd, page_size, n_pages, scale, window, 1, stream, true, firsts, n_rows, softcap);
+}
+FL_RECORDABLE(fl_attn_decode_items_capped)
 
 // ---- the same without any allocation: the splits' partial results go to an array that is part of
 // the library's image on every GPU.  `scratch` is a host-side stand-in for that array, not a device

@@ -44,7 +44,7 @@ template <int HDP, int QT, int NS>
 __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, PagedCache cache,
     const int* __restrict__ tiles, const int* __restrict__ positions,
-    const int* __restrict__ block_table, int max_blocks, int nh, float scale_log2e, int window,
+    const int* __restrict__ block_table, int max_blocks, int nh, float scale_log2e, float cap_raw, int window,
     int log2_ps, int mirror_from, float* __restrict__ part_o, float* __restrict__ part_ml) {
     constexpr int QS = HDP / 32;              // k-steps of the score product
     constexpr int DT = HDP / 16;              // tiles of head dims in the output
@@ -272,6 +272,18 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
             // chunk, a base almost never after the first ones; and whether any base has to move
             // is a vote of the lanes over their own scores, so the usual chunk needs no exchange
             // between lanes at all.
+            if (cap_raw > 0.f) {
+                // scores capped smoothly: in raw units s <- c tanh(s / c) with c = cap / scale, so that the
+                // scaled score is cap * tanh(scale s / cap) and everything below stays as it is
+                const float inv_cap = 1.0f / cap_raw;
+#pragma unroll
+                for (int t = 0; t < QT; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        sa[half][t][r] = cap_raw * tanhf(sa[half][t][r] * inv_cap);
+                        sb[half][t][r] = cap_raw * tanhf(sb[half][t][r] * inv_cap);
+                    }
+            }
             if (need_mask) {
 #pragma unroll
                 for (int t = 0; t < QT; ++t)
@@ -385,7 +397,7 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
 template <int HDP, int QT, int NS>
 static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
                                const int* tiles, const int* positions, const int* block_table, int max_blocks,
-                               int nh, float scale_log2e, int window, int log2_ps, float* part_o, float* part_ml, int lds_pages) {
+                               int nh, float scale_log2e, float cap_raw, int window, int log2_ps, float* part_o, float* part_ml, int lds_pages) {
     // blocks that the chip holds at one time: one or two per compute unit
     const int units = fl_units();
     const int total = (int)(grid.x * grid.y * grid.z);
@@ -402,23 +414,23 @@ static void launch_prefill_one(dim3 grid, hipStream_t stream, const bf16_t* q, b
                                   min(RING + PF_MAX_PAGES * (int)sizeof(int), PF_LDS_BYTES));
         configured = true;
     }
-    kern<<<grid, 256, lds, stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, mirror_from, part_o, part_ml);
+    kern<<<grid, 256, lds, stream>>>(q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, cap_raw, window, log2_ps, mirror_from, part_o, part_ml);
 }
 
 template <int HDP, int NS>
 static void launch_prefill(int qt, dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* out, PagedCache c,
                            const int* tiles, const int* positions, const int* block_table, int max_blocks, int nh,
-                           float scale_log2e, int window, int log2_ps, float* part_o, float* part_ml, int lds_pages) {
+                           float scale_log2e, float cap_raw, int window, int log2_ps, float* part_o, float* part_ml, int lds_pages) {
     if constexpr (HDP <= 64) {            // four heads per wave only where two blocks still fit a compute unit
         if (qt == 4) {
-            launch_prefill_one<HDP, 4, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml, lds_pages);
+            launch_prefill_one<HDP, 4, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, cap_raw, window, log2_ps, part_o, part_ml, lds_pages);
             return;
         }
     }
     if (qt >= 2)
-        launch_prefill_one<HDP, 2, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml, lds_pages);
+        launch_prefill_one<HDP, 2, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, cap_raw, window, log2_ps, part_o, part_ml, lds_pages);
     else
-        launch_prefill_one<HDP, 1, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, window, log2_ps, part_o, part_ml, lds_pages);
+        launch_prefill_one<HDP, 1, NS>(grid, stream, q, out, c, tiles, positions, block_table, max_blocks, nh, scale_log2e, cap_raw, window, log2_ps, part_o, part_ml, lds_pages);
 }
 
 // Query heads per wave (QT, a divisor of the group size) and parts of the keys for a batch of n_tiles
@@ -555,11 +567,11 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
 // tiles[n_tiles][4] = (row of the request in the block table, first row, rows (at most 64), index of
 // the first row among all rows of tiles).  n_split > 1 (fl_attn_prefill_splits): the keys are split,
 // part_o and part_ml hold fl_attn_prefill_workspace floats.
-extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base, const int* tiles,
+static int attn_prefill_launch(const void* q, void* out, const void* cache_base, const int* tiles,
                                int n_tiles, const int* positions, const int* block_table,
                                int max_blocks, int nh, int nkv, int hd, int page_size, int n_pages,
                                float scale, int window, int qt_hint, float* part_o, float* part_ml, int n_split,
-                               hipStream_t stream) {
+                               float softcap, hipStream_t stream) {
     FL_CHECK(n_tiles >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_prefill: bad head counts %d/%d", nh, nkv);
     FL_CHECK(hd > 0 && hd <= 256 && hd % 8 == 0, "attn_prefill: head size %d must be a multiple of 8 up to 256", hd);
     FL_CHECK(page_size >= 8 && (page_size & (page_size - 1)) == 0,
@@ -583,10 +595,11 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     const int qt = pf_heads_per_wave(n_tiles, nh, nkv, hd, qt_hint, n_split);
     dim3 grid(n_tiles, nkv * (G / qt), n_split);
     const float sl = scale * 1.4426950408889634f;
+    const float cap_raw = softcap > 0.f ? softcap / scale : 0.f;
     // a ring of two stages: two blocks then fit a compute unit (three stages were no faster)
 #define FL_PF(HDP_)                                                                                            \
     launch_prefill<HDP_, 2>(qt, grid, stream, (const bf16_t*)q, (bf16_t*)out, c, tiles, positions, block_table, \
-                            max_blocks, nh, sl, window, log2_ps, part_o, part_ml, lds_pages)
+                            max_blocks, nh, sl, cap_raw, window, log2_ps, part_o, part_ml, lds_pages)
     switch (hdp) {
         case 32: FL_PF(32); break;
         case 64: FL_PF(64); break;
@@ -607,4 +620,25 @@ extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base,
     }
     return 0;
 }
+
+extern "C" int fl_attn_prefill(const void* q, void* out, const void* cache_base, const int* tiles,
+                               int n_tiles, const int* positions, const int* block_table,
+                               int max_blocks, int nh, int nkv, int hd, int page_size, int n_pages,
+                               float scale, int window, int qt_hint, float* part_o, float* part_ml, int n_split,
+                               hipStream_t stream) {
+    return attn_prefill_launch(q, out, cache_base, tiles, n_tiles, positions, block_table, max_blocks, nh, nkv, hd, page_size,
+                               n_pages, scale, window, qt_hint, part_o, part_ml, n_split, 0.f, stream);
+}
 FL_RECORDABLE(fl_attn_prefill)
+
+// the same with the scores capped: score <- softcap * tanh(score / softcap) before the softmax (softcap > 0)
+extern "C" int fl_attn_prefill_capped(const void* q, void* out, const void* cache_base, const int* tiles,
+                                      int n_tiles, const int* positions, const int* block_table,
+                                      int max_blocks, int nh, int nkv, int hd, int page_size, int n_pages,
+                                      float scale, int window, float softcap, int qt_hint, float* part_o, float* part_ml,
+                                      int n_split, hipStream_t stream) {
+    FL_CHECK(softcap >= 0.f, "attn_prefill: negative cap");
+    return attn_prefill_launch(q, out, cache_base, tiles, n_tiles, positions, block_table, max_blocks, nh, nkv, hd, page_size,
+                               n_pages, scale, window, qt_hint, part_o, part_ml, n_split, softcap, stream);
+}
+FL_RECORDABLE(fl_attn_prefill_capped)

@@ -1,0 +1,288 @@
+// Linear recurrences with a matrix state per head, token by token, and what prepares their inputs.
+//
+// fl_linear_scan: per request and head the state S [D][Dv] (float, in the request's slot between
+// steps, zero when the slot is claimed).  For every token, with a decay g (one per head, or one per
+// token and head), q and k of the head's query/key head and v of the head:
+//     S <- g S
+//     u = beta (v - S^T k)     (the delta rule; without beta: u = v)
+//     S <- S + k u^T
+//     o = S^T q                (the read-out sees the token's own write)
+// The walk IS the recurrence, so a prompt cut anywhere leaves the same state and the same outputs.
+//
+// fl_conv_prepare: a short causal convolution over time per channel with silu behind it, for the
+// channels of q, k and v side by side; the inputs of the last taps - 1 tokens of a request live in
+// its slot (zeros before its start).  Then q and k are made unit vectors per head (q also times a
+// factor), and the decay and write strength of every (token, head) are formed:
+//     g = exp(-exp(A_log) softplus(a + dt_bias)),  beta = sigmoid(b).
+// fl_conv_state_update moves the window of kept inputs on, after every block of the first has read it.
+//
+// fl_rotate_scale: rotation of the first dims of every head of two float row sets (q and k of a
+// mixer that keeps no keys), each times a factor of its own afterwards.
+#include "common.h"
+#include "api.h"
+#include "recordable.h"
+#include "lanes.h"
+
+#define LS_GROUP 16          // threads that share a column of S; they own the rows d = g, g + 16, ...
+#define LS_COLS 16           // columns of S per block
+#define LS_MAX_ROWS 32       // rows per thread: D <= LS_GROUP * LS_MAX_ROWS
+#define LS_MAX_TAPS 16
+
+// Block = (columns j0 .. j0 + 15, head, request); thread (g, c) holds S[d][j0 + c] for its rows d.
+// State of a head: S column by column, S[d][j] at j * D + d.
+template <int RPT, bool DELTA>
+__global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
+    const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk, const float* __restrict__ v, int ldv,
+    const float* __restrict__ head_decay, const float* __restrict__ tok_decay, const float* __restrict__ beta, int ldg,
+    float* __restrict__ state, size_t slot_stride, const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
+    const int* __restrict__ seq_slots, float* __restrict__ out, int H, int G, int D, int Dv, int run) {
+    const int g = threadIdx.x & (LS_GROUP - 1), c = threadIdx.x / LS_GROUP;
+    const int j = blockIdx.x * LS_COLS + c, head = blockIdx.y, s = blockIdx.z;
+    const int qk_head = head / (H / G);
+    const bool live = j < Dv;
+    const int start = seq_q_start[s], len = seq_q_len[s];
+    float* st = state + (size_t)seq_slots[s] * slot_stride + (size_t)head * D * Dv;
+    float S[RPT];
+#pragma unroll
+    for (int u = 0; u < RPT; ++u) {
+        const int d = g + LS_GROUP * u;
+        S[u] = (live && d < D) ? st[(size_t)j * D + d] : 0.f;
+    }
+    const float fixed = head_decay ? head_decay[head] : 1.f;
+    // the step's tokens come through LDS a run at a time: one trip to memory per run, not one per token
+    extern __shared__ float ls_smem[];
+    float* qs = ls_smem;                          // [run][D]
+    float* ks = qs + (size_t)run * D;             // [run][D]
+    float* vs = ks + (size_t)run * D;             // [run][16]
+    float* fs = vs + (size_t)run * LS_COLS;       // [run][2]: decay, beta
+    for (int t0 = 0; t0 < len; t0 += run) {
+        const int cnt = min(run, len - t0);
+        __syncthreads();
+        for (int e = threadIdx.x; e < cnt * D; e += LS_GROUP * LS_COLS) {
+            const int tt = e / D, d = e - tt * D;
+            qs[e] = q[(size_t)(start + t0 + tt) * ldq + qk_head * D + d];
+            ks[e] = k[(size_t)(start + t0 + tt) * ldk + qk_head * D + d];
+        }
+        for (int e = threadIdx.x; e < cnt * LS_COLS; e += LS_GROUP * LS_COLS) {
+            const int tt = e / LS_COLS, jj = blockIdx.x * LS_COLS + (e - tt * LS_COLS);
+            vs[e] = jj < Dv ? v[(size_t)(start + t0 + tt) * ldv + head * Dv + jj] : 0.f;
+        }
+        for (int tt = threadIdx.x; tt < cnt; tt += LS_GROUP * LS_COLS) {
+            fs[2 * tt] = tok_decay ? tok_decay[(size_t)(start + t0 + tt) * ldg + head] : fixed;
+            fs[2 * tt + 1] = DELTA ? beta[(size_t)(start + t0 + tt) * ldg + head] : 1.f;
+        }
+        __syncthreads();
+        for (int tt = 0; tt < cnt; ++tt) {
+            const float decay = fs[2 * tt];
+            float uv = vs[tt * LS_COLS + c];
+            float kr[RPT];
+#pragma unroll
+            for (int u = 0; u < RPT; ++u) {
+                const int d = g + LS_GROUP * u;
+                kr[u] = d < D ? ks[tt * D + d] : 0.f;
+                S[u] *= decay;
+            }
+            if (DELTA) {
+                float seen = 0.f;
+#pragma unroll
+                for (int u = 0; u < RPT; ++u) seen = fmaf(S[u], kr[u], seen);
+                uv = fs[2 * tt + 1] * (uv - row_sum16(seen));
+            }
+            float num = 0.f;
+#pragma unroll
+            for (int u = 0; u < RPT; ++u) {
+                const int d = g + LS_GROUP * u;
+                S[u] = fmaf(kr[u], uv, S[u]);
+                num = fmaf(S[u], d < D ? qs[tt * D + d] : 0.f, num);
+            }
+            num = row_sum16(num);                                  // the 16 threads of a column are a row of lanes
+            if (live && g == 0) out[((size_t)(start + t0 + tt) * H + head) * Dv + j] = num;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < RPT; ++u) {
+        const int d = g + LS_GROUP * u;
+        if (live && d < D) st[(size_t)j * D + d] = S[u];
+    }
+}
+
+extern "C" int fl_linear_scan_max_dim(void) { return LS_GROUP * LS_MAX_ROWS; }
+
+extern "C" int fl_linear_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
+                              const float* head_decay, const float* tok_decay, const float* beta, int ldg, float* state,
+                              long slot_stride, const int* seq_q_start, const int* seq_q_len, const int* seq_slots,
+                              float* out, int n_seqs, int H, int G, int D, int Dv, hipStream_t stream) {
+    FL_CHECK(n_seqs >= 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && Dv > 0, "linear_scan: bad sizes");
+    FL_CHECK(D <= LS_GROUP * LS_MAX_ROWS, "linear_scan: %d key dims per head, at most %d", D, LS_GROUP * LS_MAX_ROWS);
+    FL_CHECK(ldq >= G * D && ldk >= G * D && ldv >= H * Dv, "linear_scan: rows narrower than their heads");
+    FL_CHECK(!head_decay != !tok_decay, "linear_scan: one decay per head or one per token and head, not both or none");
+    FL_CHECK((!tok_decay && !beta) || ldg >= H, "linear_scan: gate rows %d wide for %d heads", ldg, H);
+    FL_CHECK(slot_stride >= (long)H * D * Dv, "linear_scan: a slot of %ld floats does not hold %d heads", slot_stride, H);
+    if (n_seqs == 0) return 0;
+    FL_CHECK(n_seqs <= 65535 && H <= 65535, "linear_scan: %d requests of %d heads are more than one grid takes", n_seqs, H);
+    dim3 grid(ceil_div(Dv, LS_COLS), H, n_seqs);
+    const int rpt = ceil_div(D, LS_GROUP);
+    int run = (60 * 1024) / ((2 * D + LS_COLS + 2) * (int)sizeof(float));
+    run = run > 32 ? 32 : (run < 1 ? 1 : run);
+    const size_t lds = (size_t)run * (2 * D + LS_COLS + 2) * sizeof(float);
+#define FL_LS2(R, DELTA)                                                                                              \
+    linear_scan_kernel<R, DELTA><<<grid, LS_GROUP * LS_COLS, lds, stream>>>(q, ldq, k, ldk, v, ldv, head_decay, tok_decay, beta, \
+                                                                            ldg, state, (size_t)slot_stride, seq_q_start,        \
+                                                                            seq_q_len, seq_slots, out, H, G, D, Dv, run)
+#define FL_LS(R)             \
+    do {                     \
+        if (beta) FL_LS2(R, true); \
+        else FL_LS2(R, false);     \
+    } while (0)
+    if (rpt <= 1) FL_LS(1);
+    else if (rpt <= 2) FL_LS(2);
+    else if (rpt <= 4) FL_LS(4);
+    else if (rpt <= 8) FL_LS(8);
+    else if (rpt <= 16) FL_LS(16);
+    else FL_LS(LS_MAX_ROWS);
+#undef FL_LS
+#undef FL_LS2
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_linear_scan)
+
+// ------------------------------------------------------------------ short convolution, unit vectors, gates
+struct ConvPrepare {
+    const float* proj; int ld; int col0, col_b, col_a;
+    const float* conv_w;                 // [C][taps], the last column is the current token's
+    const float* a_log; const float* dt_bias;
+    const float* conv_state; size_t slot_stride;      // per slot [taps - 1][C]: the inputs before the step, oldest first
+    const int* tok_seq; const int* seq_q_start; const int* seq_slots;
+    float* prep; float* gates;           // [n][C], [n][2 H]: decay, beta
+    int G, H, D, Dv, taps;
+    float q_scale, unit_eps;
+};
+
+__global__ __launch_bounds__(256) void conv_prepare_kernel(ConvPrepare a) {
+    const int token = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int C = 2 * a.G * a.D + a.H * a.Dv, taps = a.taps;
+    const int s = a.tok_seq[token];
+    const int back = token - a.seq_q_start[s];            // tokens of the request in this step before this one
+    const float* hist = a.conv_state + (size_t)a.seq_slots[s] * a.slot_stride;
+    float* dst = a.prep + (size_t)token * C;
+    for (int c = threadIdx.x; c < C; c += 256) {
+        float y = 0.f;
+        for (int jj = taps - 1; jj >= 0; --jj) {          // oldest input first
+            const float x = jj <= back ? a.proj[(size_t)(token - jj) * a.ld + a.col0 + c]
+                                       : hist[(size_t)(taps - 1 - (jj - back)) * C + c];
+            y = fmaf(a.conv_w[(size_t)c * taps + (taps - 1 - jj)], x, y);
+        }
+        dst[c] = y / (1.0f + expf(-y));
+    }
+    if (threadIdx.x < a.H) {
+        const int h = threadIdx.x;
+        const float* row = a.proj + (size_t)token * a.ld;
+        const float z = row[a.col_a + h] + a.dt_bias[h];
+        const float sp = z > 20.f ? z : log1pf(expf(z));
+        a.gates[(size_t)token * 2 * a.H + h] = expf(-expf(a.a_log[h]) * sp);
+        a.gates[(size_t)token * 2 * a.H + a.H + h] = 1.0f / (1.0f + expf(-row[a.col_b + h]));
+    }
+    __syncthreads();
+    // q heads, then k heads: unit vectors
+    for (int head = wave; head < 2 * a.G; head += 4) {
+        float* x = dst + (size_t)head * a.D;
+        float ss = 0.f;
+        for (int d = lane; d < a.D; d += 64) ss = fmaf(x[d], x[d], ss);
+        const float f = (head < a.G ? a.q_scale : 1.f) / sqrtf(wave_sum(ss) + a.unit_eps);
+        for (int d = lane; d < a.D; d += 64) x[d] *= f;
+    }
+}
+
+// per (request, channel): the kept inputs move on by the request's tokens of this step
+__global__ __launch_bounds__(256) void conv_state_update_kernel(const float* __restrict__ proj, int ld, int col0, int C, int taps,
+                                                                float* __restrict__ conv_state, size_t slot_stride,
+                                                                const int* __restrict__ seq_q_start,
+                                                                const int* __restrict__ seq_q_len,
+                                                                const int* __restrict__ seq_slots) {
+    const int c = blockIdx.x * 256 + threadIdx.x, s = blockIdx.y;
+    if (c >= C) return;
+    const int start = seq_q_start[s], len = seq_q_len[s], keep = taps - 1;
+    float* hist = conv_state + (size_t)seq_slots[s] * slot_stride;
+    float old[LS_MAX_TAPS];
+#pragma unroll
+    for (int r = 0; r < LS_MAX_TAPS; ++r) old[r] = r < keep ? hist[(size_t)r * C + c] : 0.f;
+#pragma unroll
+    for (int r = 0; r < LS_MAX_TAPS; ++r) {
+        if (r >= keep) break;
+        const int rel = len - keep + r;                    // which of this step's tokens, or (negative) an older one
+        hist[(size_t)r * C + c] = rel >= 0 ? proj[(size_t)(start + rel) * ld + col0 + c] : old[r + len];
+    }
+}
+
+extern "C" int fl_conv_max_taps(void) { return LS_MAX_TAPS; }
+
+extern "C" int fl_conv_prepare(const float* proj, int ld, int col0, int col_b, int col_a, const float* conv_w,
+                               const float* a_log, const float* dt_bias, float* conv_state, long slot_stride,
+                               const int* tok_seq, const int* seq_q_start, const int* seq_q_len, const int* seq_slots,
+                               float* prep, float* gates, int n, int n_seqs, int G, int H, int D, int Dv, int taps,
+                               float q_scale, float unit_eps, hipStream_t stream) {
+    FL_CHECK(n >= 0 && n_seqs >= 0 && G > 0 && H > 0 && D > 0 && Dv > 0, "conv_prepare: bad sizes");
+    FL_CHECK(taps >= 1 && taps <= LS_MAX_TAPS, "conv_prepare: %d taps, at most %d", taps, LS_MAX_TAPS);
+    FL_CHECK(H <= 256, "conv_prepare: %d heads, at most 256", H);
+    const int C = 2 * G * D + H * Dv;
+    FL_CHECK(ld >= col0 + C && ld >= col_b + H && ld >= col_a + H, "conv_prepare: columns beyond rows %d wide", ld);
+    FL_CHECK(slot_stride >= (long)(taps - 1) * C, "conv_prepare: a slot of %ld floats does not hold %d inputs of %d channels",
+             slot_stride, taps - 1, C);
+    if (n == 0) return 0;
+    FL_CHECK(n_seqs <= 65535, "conv_prepare: %d requests are more than one grid takes", n_seqs);
+    ConvPrepare a{proj, ld, col0, col_b, col_a, conv_w, a_log, dt_bias, conv_state, (size_t)slot_stride, tok_seq, seq_q_start,
+                  seq_slots, prep, gates, G, H, D, Dv, taps, q_scale, unit_eps};
+    conv_prepare_kernel<<<n, 256, 0, stream>>>(a);
+    FL_LAUNCH_CHECK();
+    if (taps > 1 && n_seqs > 0) {
+        dim3 grid(ceil_div(C, 256), n_seqs);
+        conv_state_update_kernel<<<grid, 256, 0, stream>>>(proj, ld, col0, C, taps, conv_state, (size_t)slot_stride, seq_q_start,
+                                                           seq_q_len, seq_slots);
+        FL_LAUNCH_CHECK();
+    }
+    return 0;
+}
+FL_RECORDABLE(fl_conv_prepare)
+
+// ------------------------------------------------------------------ rotation of float rows
+// out[t][h][d] of two row sets a (H heads) and b (H heads), both D wide per head: the first rot dims turned
+// by the step's table, pairs (i, i + rot/2) or (2i, 2i + 1); a times scale_a, b times scale_b afterwards.
+__global__ __launch_bounds__(256) void rotate_scale_kernel(const float* __restrict__ proj, int ld, int col_a, int col_b,
+                                                           const float2* __restrict__ cs, int rot, int interleaved, float scale_a,
+                                                           float scale_b, float* __restrict__ out_a, float* __restrict__ out_b,
+                                                           int H, int D) {
+    const size_t token = blockIdx.x;
+    const int half = rot >> 1;
+    for (int e = threadIdx.x; e < 2 * H * D; e += 256) {
+        const bool is_b = e >= H * D;
+        const int f = is_b ? e - H * D : e;
+        const int h = f / D, d = f - h * D;
+        const float* src = proj + token * ld + (is_b ? col_b : col_a) + h * D;
+        float v = src[d];
+        if (d < rot) {
+            int i, partner;
+            bool first;
+            if (interleaved) { i = d >> 1; first = !(d & 1); partner = d ^ 1; }
+            else { first = d < half; i = first ? d : d - half; partner = first ? d + half : d - half; }
+            const float2 c = cs[token * half + i];
+            const float o = src[partner];
+            v = first ? v * c.x - o * c.y : v * c.x + o * c.y;
+        }
+        (is_b ? out_b : out_a)[token * H * D + f] = v * (is_b ? scale_b : scale_a);
+    }
+}
+
+extern "C" int fl_rotate_scale(const float* proj, int ld, int col_a, int col_b, const float* cs, int rot, int interleaved,
+                               float scale_a, float scale_b, float* out_a, float* out_b, int n, int H, int D,
+                               hipStream_t stream) {
+    FL_CHECK(n >= 0 && H > 0 && D > 0, "rotate_scale: bad sizes");
+    FL_CHECK(rot >= 0 && rot <= D && rot % 2 == 0 && (rot == 0 || cs), "rotate_scale: rotated dims %d of head %d", rot, D);
+    FL_CHECK(ld >= col_a + H * D && ld >= col_b + H * D, "rotate_scale: columns beyond rows %d wide", ld);
+    if (n == 0) return 0;
+    rotate_scale_kernel<<<n, 256, 0, stream>>>(proj, ld, col_a, col_b, (const float2*)cs, rot, interleaved, scale_a, scale_b,
+                                               out_a, out_b, H, D);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_rotate_scale)

@@ -13,25 +13,11 @@
 #include "common.h"
 #include "api.h"
 #include "recordable.h"
+#include "lanes.h"
 
 #define ML_GROUP 16          // threads that share a column of S; they own the rows d = g, g + 16, ...
 #define ML_COLS 16           // columns of S per block
 #define ML_MAX_ROWS 32       // rows per thread: D <= ML_GROUP * ML_MAX_ROWS
-
-// v of the lane `n` places further round its row of 16 lanes (a data-parallel move between neighbouring lanes:
-// no trip through LDS, which is what a shuffle costs)
-template <int N>
-__device__ __forceinline__ float row_rotated(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + N, 0xf, 0xf, false));
-}
-// the sum over the 16 lanes of a row, in every lane
-__device__ __forceinline__ float row_sum16(float v) {
-    v += row_rotated<8>(v);
-    v += row_rotated<4>(v);
-    v += row_rotated<2>(v);
-    v += row_rotated<1>(v);
-    return v;
-}
 
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
@@ -192,12 +178,13 @@ extern "C" int fl_mlstm_scan(const float* proj, int ld, int col_q, int col_k, in
 FL_RECORDABLE(fl_mlstm_scan)
 
 // ------------------------------------------------------------------ unit norm per head, gain, gate
-// out[t][h][:] = o / sqrt(mean(o^2) + eps) * w[h][:] * sigmoid(gate[t][gate_col0 + h * Dv + :]),
-// o = x[t][h][:] (float).  One wave per (token, head).
+// out[t][h][:] = o / sqrt(mean(o^2) + eps) * w[h][:] * g(gate[t][gate_col0 + h * Dv + :]),
+// o = x[t][h][:] (float); g the sigmoid (gate_kind 1) or silu (2).  One wave per (token, head).
 template <typename T>
 __global__ __launch_bounds__(256) void headnorm_gate_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                             const float* __restrict__ gate, int ldg, int gate_col0,
-                                                            T* __restrict__ out, int n_heads_total, int H, int Dv, float eps) {
+                                                            T* __restrict__ out, int n_heads_total, int H, int Dv, float eps,
+                                                            int gate_kind) {
     const int unit = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (unit >= n_heads_total) return;
     const int t = unit / H, h = unit - t * H;
@@ -207,23 +194,27 @@ __global__ __launch_bounds__(256) void headnorm_gate_kernel(const float* __restr
     const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)Dv + eps);
     for (int i = lane; i < Dv; i += 64) {
         float v = xr[i] * inv * (w ? w[h * Dv + i] : 1.0f);
-        if (gate) v *= 1.0f / (1.0f + expf(-gate[(size_t)t * ldg + gate_col0 + h * Dv + i]));
+        if (gate) {
+            const float z = gate[(size_t)t * ldg + gate_col0 + h * Dv + i];
+            v *= (gate_kind == 2 ? z : 1.0f) / (1.0f + expf(-z));
+        }
         out[(size_t)unit * Dv + i] = from_f32<T>(v);
     }
 }
 
 extern "C" int fl_headnorm_gate(const float* x, const float* w, const float* gate, int ldg, int gate_col0, void* out,
-                                int out_dtype, int n, int H, int Dv, float eps, hipStream_t stream) {
+                                int out_dtype, int n, int H, int Dv, float eps, int gate_kind, hipStream_t stream) {
     FL_CHECK(n >= 0 && H > 0 && Dv > 0, "headnorm_gate: bad sizes");
+    FL_CHECK(gate_kind == 1 || gate_kind == 2, "headnorm_gate: gate %d (1 sigmoid, 2 silu)", gate_kind);
     FL_CHECK(!gate || ldg >= gate_col0 + H * Dv, "headnorm_gate: gate columns beyond rows %d wide", ldg);
     if (n == 0) return 0;
     const long units = (long)n * H;
     FL_CHECK(units < (1L << 31), "headnorm_gate: too many rows");
     const int blocks = (int)((units + 3) / 4);
     if (out_dtype == FL_F32)
-        headnorm_gate_kernel<float><<<blocks, 256, 0, stream>>>(x, w, gate, ldg, gate_col0, (float*)out, (int)units, H, Dv, eps);
+        headnorm_gate_kernel<float><<<blocks, 256, 0, stream>>>(x, w, gate, ldg, gate_col0, (float*)out, (int)units, H, Dv, eps, gate_kind);
     else if (out_dtype == FL_BF16)
-        headnorm_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, w, gate, ldg, gate_col0, (bf16_t*)out, (int)units, H, Dv, eps);
+        headnorm_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, w, gate, ldg, gate_col0, (bf16_t*)out, (int)units, H, Dv, eps, gate_kind);
     else
         FL_CHECK(false, "headnorm_gate: unknown dtype %d", out_dtype);
     FL_LAUNCH_CHECK();

@@ -428,7 +428,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void attn_plain_kernel(
     const T* __restrict__ q, T* __restrict__ out, PagedCache cache,
     const int* __restrict__ positions, const int* __restrict__ tok_seq,
-    const int* __restrict__ block_table, int max_blocks, int nh, float scale, int window) {
+    const int* __restrict__ block_table, int max_blocks, int nh, float scale, int window, float softcap) {
     __shared__ float s_m[4], s_l[4];
     __shared__ float s_acc[4][FL_PLAIN_MAX_HD];
     const int token = blockIdx.x, head = blockIdx.y;
@@ -460,7 +460,8 @@ __global__ __launch_bounds__(256) void attn_plain_kernel(
             const int d = lane + 64 * j;
             if (d < hd) part = fmaf(qv[j], to_f32(kr[d]), part);
         }
-        const float s = wave_sum(part) * scale;
+        float s = wave_sum(part) * scale;
+        if (softcap > 0.f) s = softcap * tanhf(s / softcap);          // scores capped smoothly at +-softcap
         const float m_new = fmaxf(m, s);
         const float corr = expf(m - m_new);
         const float pe = expf(s - m_new);
@@ -505,10 +506,10 @@ __global__ __launch_bounds__(256) void attn_plain_kernel(
 // The largest head size any attention kernel of the library takes (the plain kernel keeps a head in LDS).
 extern "C" int fl_attn_max_head_dim(void) { return FL_PLAIN_MAX_HD; }
 
-extern "C" int fl_attn_plain(const void* q, void* out, const void* cache_base, int dtype,
+static int attn_plain_launch(const void* q, void* out, const void* cache_base, int dtype,
                              const int* positions, const int* tok_seq, const int* block_table,
                              int max_blocks, int n, int nh, int nkv, int hd, int page_size,
-                             int n_pages, float scale, int window, hipStream_t stream) {
+                             int n_pages, float scale, int window, float softcap, hipStream_t stream) {
     FL_CHECK(n >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn: bad head counts %d/%d", nh, nkv);
     FL_CHECK(hd > 0 && hd <= FL_PLAIN_MAX_HD, "attn: head size %d not in 1..%d", hd, FL_PLAIN_MAX_HD);
     FL_CHECK(window >= 0, "attn: negative window");
@@ -516,15 +517,34 @@ extern "C" int fl_attn_plain(const void* q, void* out, const void* cache_base, i
     PagedCache c{(void*)cache_base, nkv, page_size, hd, n_pages};
     dim3 grid(n, nh);
     if (dtype == FL_F32)
-        attn_plain_kernel<float><<<grid, 256, 0, stream>>>((const float*)q, (float*)out, c, positions, tok_seq, block_table, max_blocks, nh, scale, window);
+        attn_plain_kernel<float><<<grid, 256, 0, stream>>>((const float*)q, (float*)out, c, positions, tok_seq, block_table, max_blocks, nh, scale, window, softcap);
     else if (dtype == FL_BF16)
-        attn_plain_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, c, positions, tok_seq, block_table, max_blocks, nh, scale, window);
+        attn_plain_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, c, positions, tok_seq, block_table, max_blocks, nh, scale, window, softcap);
     else
         FL_CHECK(false, "attn: unknown dtype %d", dtype);
     FL_LAUNCH_CHECK();
     return 0;
 }
+
+extern "C" int fl_attn_plain(const void* q, void* out, const void* cache_base, int dtype,
+                             const int* positions, const int* tok_seq, const int* block_table,
+                             int max_blocks, int n, int nh, int nkv, int hd, int page_size,
+                             int n_pages, float scale, int window, hipStream_t stream) {
+    return attn_plain_launch(q, out, cache_base, dtype, positions, tok_seq, block_table, max_blocks, n, nh, nkv, hd, page_size,
+                             n_pages, scale, window, 0.f, stream);
+}
 FL_RECORDABLE(fl_attn_plain)
+
+// the same with the scores capped: score <- softcap * tanh(score / softcap) before the softmax (softcap > 0)
+extern "C" int fl_attn_plain_capped(const void* q, void* out, const void* cache_base, int dtype,
+                                    const int* positions, const int* tok_seq, const int* block_table,
+                                    int max_blocks, int n, int nh, int nkv, int hd, int page_size,
+                                    int n_pages, float scale, int window, float softcap, hipStream_t stream) {
+    FL_CHECK(softcap >= 0.f, "attn: negative cap");
+    return attn_plain_launch(q, out, cache_base, dtype, positions, tok_seq, block_table, max_blocks, n, nh, nkv, hd, page_size,
+                             n_pages, scale, window, softcap, stream);
+}
+FL_RECORDABLE(fl_attn_plain_capped)
 
 // ------------------------------------------------------------------ SiLU gate
 // out[r, i] = silu(gu[r, i]) * gu[r, I + i], silu(g) = g / (1 + exp(-g)), all in float.

@@ -1,0 +1,137 @@
+// What stands between the joined q/k/v projection of a softmax-attention mixer and attention itself,
+// for mixers whose queries and keys are normed and whose heads differ in key and value size:
+//   * a norm over the WHOLE projection of q (and of k) with a gain per value, before rotation
+//     (x / sqrt(mean(x^2) + eps) * w over all heads at once), or none;
+//   * rotation of the first `rot` dims of every head from the step's table of cosines and sines, pairs
+//     (i, i + rot/2) ("half") or (2i, 2i + 1) ("interleaved");
+//   * every head of q and k divided by its root mean square after rotation (no gain), or not;
+//   * values blended with those an earlier layer made for the same token,
+//     v <- (1 - lambda) v + lambda v_first, or kept as that first layer's for later ones;
+//   * q stored for the attention kernels, k and v stored into the paged cache at the token's position.
+// Heads are stored `hdp` wide (hdp >= max(D, Dv)): keys are padded with zeros behind D, values behind
+// Dv, queries behind D, so that attention kernels of one head size serve key and value sizes that differ.
+// The projection arrives in float; everything here is float, only the stores are in the cache's type.
+#include "common.h"
+#include "api.h"
+#include "recordable.h"
+
+struct QkvPrepare {
+    const float* proj; int ld; int col_q, col_k, col_v;
+    const int* positions; const int* tok_seq; const int* block_table; int max_blocks;
+    int nh, D, Dv, hdp;
+    int rot, interleaved; const float2* cs;
+    const float* qnorm_w; const float* knorm_w; int head_norm; float eps;
+    float* v_first; int vmix_mode; const float* lambda;
+    int write_cache;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __restrict__ q_out, PagedCache cache) {
+    __shared__ float lds[8];
+    const int token = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nh = a.nh, nkv = cache.n_kv_heads, D = a.D, Dv = a.Dv, hdp = a.hdp;
+    const float* row = a.proj + (size_t)token * a.ld;
+    float inv_q = 1.f, inv_k = 1.f;
+    if (a.qnorm_w) {
+        float sq = 0.f, sk = 0.f;
+        for (int i = threadIdx.x; i < nh * D; i += 256) sq = fmaf(row[a.col_q + i], row[a.col_q + i], sq);
+        for (int i = threadIdx.x; i < nkv * D; i += 256) sk = fmaf(row[a.col_k + i], row[a.col_k + i], sk);
+        inv_q = 1.0f / sqrtf(block_sum<4>(sq, lds) / (float)(nh * D) + a.eps);
+        inv_k = 1.0f / sqrtf(block_sum<4>(sk, lds + 4) / (float)(nkv * D) + a.eps);
+    }
+    const int pos = a.positions[token];
+    int page = -1, prow = 0;
+    if (a.write_cache) {
+        page = a.block_table[(size_t)a.tok_seq[token] * a.max_blocks + pos / cache.page_size];
+        if (page >= cache.n_pages) page = -1;             // (padding rows of a fixed-size batch have no page)
+        prow = pos % cache.page_size;
+    }
+    const int half = a.rot >> 1;
+    // q and k heads: a wave per head, a lane per head dim (and the dims 64, 128, ... further)
+    for (int head = wave; head < nh + nkv; head += 4) {
+        const bool is_q = head < nh;
+        const int h = is_q ? head : head - nh;
+        const float* src = row + (is_q ? a.col_q : a.col_k) + h * D;
+        const float* gain = is_q ? a.qnorm_w : a.knorm_w;
+        const float inv = is_q ? inv_q : inv_k;
+        auto value = [&](int d) { return gain ? src[d] * inv * gain[h * D + d] : src[d]; };
+        float r[4];
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int d = lane + 64 * j;
+            r[j] = 0.f;
+            if (d >= D) continue;
+            float v = value(d);
+            if (d < a.rot) {
+                int i, partner;
+                bool first;
+                if (a.interleaved) { i = d >> 1; first = !(d & 1); partner = d ^ 1; }
+                else { first = d < half; i = first ? d : d - half; partner = first ? d + half : d - half; }
+                const float2 c = a.cs[(size_t)token * half + i];
+                const float o = value(partner);
+                v = first ? v * c.x - o * c.y : v * c.x + o * c.y;
+            }
+            r[j] = v;
+            ss = fmaf(v, v, ss);
+        }
+        if (a.head_norm) {
+            const float f = 1.0f / sqrtf(wave_sum(ss) / (float)D + a.eps);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) r[j] *= f;
+        }
+        if (is_q) {
+            T* dst = q_out + ((size_t)token * nh + h) * hdp;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (lane + 64 * j < hdp) dst[lane + 64 * j] = from_f32<T>(r[j]);
+        } else if (page >= 0) {
+            T* dst = (T*)cache.base + cache_k_offset(cache, page, h, prow, 0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (lane + 64 * j < hdp) dst[lane + 64 * j] = from_f32<T>(r[j]);
+        }
+    }
+    // v heads
+    const float lam = a.vmix_mode == 2 ? a.lambda[0] : 0.f;
+    for (int e = threadIdx.x; e < nkv * hdp; e += 256) {
+        const int h = e / hdp, d = e - h * hdp;
+        float v = 0.f;
+        if (d < Dv) {
+            v = row[a.col_v + h * Dv + d];
+            const size_t at = (size_t)token * nkv * Dv + h * Dv + d;
+            if (a.vmix_mode == 1) a.v_first[at] = v;
+            else if (a.vmix_mode == 2) v = (1.0f - lam) * v + lam * a.v_first[at];
+        }
+        if (page >= 0) ((T*)cache.base)[cache_v_offset(cache, page, h, prow, d)] = from_f32<T>(v);
+    }
+}
+
+extern "C" int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, int col_v, const int* positions,
+                              const int* tok_seq, const int* block_table, int max_blocks, void* q_out, void* cache_base,
+                              int dtype, int n, int nh, int nkv, int D, int Dv, int hdp, int page_size, int n_pages, int rot,
+                              int interleaved, const float* cs, const float* qnorm_w, const float* knorm_w, int head_norm,
+                              float eps, float* v_first, int vmix_mode, const float* lambda, int write_cache,
+                              hipStream_t stream) {
+    FL_CHECK(n >= 0 && nh > 0 && nkv > 0 && D > 0 && Dv > 0 && page_size > 0, "qkv_prepare: bad sizes");
+    FL_CHECK(hdp >= D && hdp >= Dv && hdp <= 256, "qkv_prepare: heads of %d and %d values stored %d wide (at most 256)", D, Dv, hdp);
+    FL_CHECK(rot >= 0 && rot <= D && rot % 2 == 0, "qkv_prepare: rotated dims %d of head %d", rot, D);
+    FL_CHECK(rot == 0 || cs, "qkv_prepare: a rotation needs the step's table of cosines and sines");
+    FL_CHECK(ld >= col_q + nh * D && ld >= col_k + nkv * D && ld >= col_v + nkv * Dv, "qkv_prepare: columns beyond rows %d wide", ld);
+    FL_CHECK(!qnorm_w == !knorm_w, "qkv_prepare: the norm over the projection needs both gains");
+    FL_CHECK(vmix_mode >= 0 && vmix_mode <= 2 && (vmix_mode == 0 || v_first) && (vmix_mode != 2 || lambda),
+             "qkv_prepare: value blending %d without its buffers", vmix_mode);
+    if (n == 0) return 0;
+    QkvPrepare a{proj, ld, col_q, col_k, col_v, positions, tok_seq, block_table, max_blocks, nh, D, Dv, hdp,
+                 rot, interleaved, (const float2*)cs, qnorm_w, knorm_w, head_norm, eps, v_first, vmix_mode, lambda, write_cache};
+    PagedCache c{cache_base, nkv, page_size, hdp, n_pages};
+    if (dtype == FL_F32)
+        qkv_prepare_kernel<float><<<n, 256, 0, stream>>>(a, (float*)q_out, c);
+    else if (dtype == FL_BF16)
+        qkv_prepare_kernel<bf16_t><<<n, 256, 0, stream>>>(a, (bf16_t*)q_out, c);
+    else
+        FL_CHECK(false, "qkv_prepare: unknown dtype %d", dtype);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_qkv_prepare)

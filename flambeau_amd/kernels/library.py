@@ -41,7 +41,7 @@ _SIGNATURES = {
     "fl_latent_attention_shared": [P, P, P, P, P, P, I, I, I, I, I, F, I, P, I, P],
     "fl_heads_matmul_mfma": [P, I, I, P, P, I, I, I, I, I, P, I, I, P],
     "fl_mlstm_scan": [P, I, I, I, I, I, I, P, P, F, F, P, P, P, P, P, P, I, I, I, I, P],
-    "fl_headnorm_gate": [P, P, P, I, I, P, I, I, I, I, F, P],
+    "fl_headnorm_gate": [P, P, P, I, I, P, I, I, I, I, F, I, P],
     "fl_moe_route": [P, I, I, I, I, I, I, I, P, P, P, P, P, I, P],
     "fl_moe_gemm": [P, I, P, P, P, P, P, I, I, I, P],
     "fl_moe_gemm_mfma": [P, P, P, P, P, P, I, I, I, I, P],
@@ -50,6 +50,16 @@ _SIGNATURES = {
     "fl_activation": [P, P, I, L, I, P],
     "fl_concat_cast": [P, P, P, I, I, I, P],
     "fl_add_rowvec": [P, P, I, I, P],
+    "fl_attn_plain_capped": [P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, F, P],
+    "fl_dyt": [P, P, P, P, P, P, P, P, I, I, I, P],
+    "fl_embed_scaled": [P, I, P, P, I, I, I, F, P],
+    "fl_gated_act": [P, P, I, I, I, I, P],
+    "fl_norm_mix": [P, P, F, P, P, F, P, I, I, F, P],
+    "fl_heads_gate": [P, I, I, P, I, I, I, P, I, I, I, P],
+    "fl_qkv_prepare": [P, I, I, I, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, I, I, I, P, P, P, I, F, P, I, P, I, P],
+    "fl_linear_scan": [P, I, P, I, P, I, P, P, P, I, P, L, P, P, P, P, I, I, I, I, I, P],
+    "fl_conv_prepare": [P, I, I, I, I, P, P, P, P, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, P],
+    "fl_rotate_scale": [P, I, I, I, P, I, I, F, F, P, P, I, I, I, P],
 }
 
 

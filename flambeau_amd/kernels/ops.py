@@ -179,17 +179,18 @@ def rope_kv_write(qkv, positions, tok_seq, block_table, q_out, cache: PagedLayer
     return q_out
 
 
-def attn_plain(q, out, cache: PagedLayerCache, positions, tok_seq, block_table, n_heads, scale, window):
+def attn_plain(q, out, cache: PagedLayerCache, positions, tok_seq, block_table, n_heads, scale, window, softcap: float = 0.0):
+    """``softcap`` > 0: scores are capped, ``softcap * tanh(score / softcap)``, before the softmax."""
     n = q.shape[0]
     hd = cache.head_dim
     dt = cache.pool.dtype
-    call("fl_attn_plain", _check(q, "attn.q", dt, (n, n_heads * hd)),
+    call("fl_attn_plain_capped" if softcap else "fl_attn_plain", _check(q, "attn.q", dt, (n, n_heads * hd)),
          _check(out, "attn.out", dt, (n, n_heads * hd)), _check(cache.pool, "attn.cache"),
          dtype_code(dt), _check(positions, "attn.positions", torch.int32, (n,)),
          _check(tok_seq, "attn.tok_seq", torch.int32, (n,)),
          _check(block_table, "attn.block_table", torch.int32, (None, None)), block_table.shape[1],
          n, n_heads, cache.n_kv_heads, hd, cache.page_size, cache.n_pages, float(scale), int(window),
-         stream_handle())
+         *((float(softcap),) if softcap else ()), stream_handle())
     return out
 
 
@@ -395,16 +396,16 @@ def mlstm_scan(proj, cols, bias_i, bias_f, cap, q_scale, state, seq_q_start, seq
     return out
 
 
-def headnorm_gate(x, weight, gate, gate_col0, out, n_heads, eps):
+def headnorm_gate(x, weight, gate, gate_col0, out, n_heads, eps, gate_kind: str = "sigmoid"):
     """Every head's slice of ``x`` (float32 ``[n, H * Dv]``) divided by its root mean square, times ``weight``
-    ``[H * Dv]``, times the sigmoid of ``gate[:, gate_col0 : gate_col0 + H * Dv]``."""
+    ``[H * Dv]``, times the sigmoid (or, ``gate_kind`` "silu", the silu) of ``gate[:, gate_col0 : gate_col0 + H * Dv]``."""
     n, HD = x.shape
     Dv = HD // n_heads
     call("fl_headnorm_gate", _check(x, "headnorm_gate.x", torch.float32),
          _check(weight, "headnorm_gate.weight", torch.float32, (HD,)) if weight is not None else None,
          _check(gate, "headnorm_gate.gate", torch.float32, (n, None)) if gate is not None else None,
          gate.shape[1] if gate is not None else 0, int(gate_col0), _check(out, "headnorm_gate.out", None, (n, HD)),
-         dtype_code(out.dtype), n, int(n_heads), Dv, float(eps), stream_handle())
+         dtype_code(out.dtype), n, int(n_heads), Dv, float(eps), {"sigmoid": 1, "silu": 2}[gate_kind], stream_handle())
     return out
 
 
@@ -497,3 +498,159 @@ def add_rowvec(x, v):
     call("fl_add_rowvec", _check(x, "add_rowvec.x", torch.float32), _check(v, "add_rowvec.v", torch.float32, (W,)), n, W,
          stream_handle())
     return x
+
+
+# ---------------------------------------------------------------- norms without statistics, gated attention, linear recurrences
+def dyt(x, alpha, weight, bias, out, delta=None, store_sum=False, rows=None):
+    """``out = tanh(alpha * (x (+ delta))) * weight + bias`` (``alpha`` a float32 scalar on the device);
+    ``store_sum`` and ``rows`` as for ``rmsnorm``."""
+    n, H = x.shape
+    px = _check(x, "dyt.x", torch.float32, (n, H))
+    pd = _check(delta, "dyt.delta", torch.float32, (n, H)) if delta is not None else None
+    pr = _check(rows, "dyt.rows", torch.int32) if rows is not None else None
+    n_out = rows.shape[0] if rows is not None else n
+    if alpha.numel() != 1:
+        raise KernelError(f"dyt.alpha: {alpha.numel()} values, one wanted")
+    call("fl_dyt", px, pd, px if store_sum and delta is not None else None, pr, _check(alpha, "dyt.alpha", torch.float32),
+         _check(weight, "dyt.weight", torch.float32, (H,)), _check(bias, "dyt.bias", torch.float32, (H,)) if bias is not None else None,
+         _check(out, "dyt.out", None, (n_out, H)), dtype_code(out.dtype), n_out, H, stream_handle())
+    return out
+
+
+def embed_scaled(table, tokens, out, scale: float):
+    V, H = table.shape
+    n = tokens.shape[0]
+    call("fl_embed_scaled", _check(table, "embed.table"), dtype_code(table.dtype), _check(tokens, "embed.tokens", torch.int32, (n,)),
+         _check(out, "embed.out", torch.float32, (n, H)), n, H, V, float(scale), stream_handle())
+    return out
+
+
+def gated_act(gu, out, kind: str):
+    """``out[r, i] = act(gu[r, i]) * gu[r, I + i]`` for float32 ``gu`` ``[n, 2 I]``."""
+    n, two_i = gu.shape
+    I = two_i // 2
+    call("fl_gated_act", _check(gu, "gated_act.gu", torch.float32), _check(out, "gated_act.out", None, (n, I)), dtype_code(out.dtype),
+         n, I, ACTIVATIONS[kind], stream_handle())
+    return out
+
+
+def norm_mix(a, weight_a, factor_a, b, weight_b, factor_b, out, eps):
+    """``out = factor_a * rmsnorm(a) * weight_a + factor_b * rmsnorm(b) * weight_b`` row by row, all float32."""
+    n, H = a.shape
+    call("fl_norm_mix", _check(a, "norm_mix.a", torch.float32), _check(weight_a, "norm_mix.weight_a", torch.float32, (H,)), float(factor_a),
+         _check(b, "norm_mix.b", torch.float32, (n, H)), _check(weight_b, "norm_mix.weight_b", torch.float32, (H,)), float(factor_b),
+         _check(out, "norm_mix.out", torch.float32, (n, H)), n, H, float(eps), stream_handle())
+    return out
+
+
+HEAD_GATES = {None: 0, "sigmoid": 1, "silu": 2}
+
+
+def heads_gate(x, head_stride, gate, gate_col0, kind, out, n_heads):
+    """``out[t, h, j] = x[t, h, j] * g(gate[t, gate_col0 + h * Dv + j])`` for ``j < Dv``; the heads of ``x`` are
+    ``head_stride`` wide (padded), those of ``out`` ``Dv``.  ``kind``: ``None``, ``sigmoid`` or ``silu``."""
+    n = x.shape[0]
+    Dv = out.shape[1] // n_heads
+    call("fl_heads_gate", _check(x, "heads_gate.x", out.dtype, (n, n_heads * head_stride)), dtype_code(x.dtype), int(head_stride),
+         _check(gate, "heads_gate.gate", torch.float32, (n, None)) if gate is not None else None,
+         gate.shape[1] if gate is not None else 0, int(gate_col0), HEAD_GATES[kind if gate is not None else None],
+         _check(out, "heads_gate.out", None, (n, n_heads * Dv)), n, int(n_heads), Dv, stream_handle())
+    return out
+
+
+def qkv_prepare(proj, cols, positions, tok_seq, block_table, q_out, cache: PagedLayerCache, n_heads, dim, vdim, rotated_dims,
+                interleaved, table, q_gain, k_gain, head_norm, eps, v_first=None, value_mix: int = 0, mix=None, write_cache=True):
+    """From the float32 rows of a joined projection (q, k, v at the columns ``cols``) to the rotated, normed
+    queries in ``q_out`` and the token's keys and values in the cache, heads stored ``cache.head_dim`` wide.
+    ``q_gain`` / ``k_gain``: gains of a norm over the whole projection of q and of k (before rotation);
+    ``head_norm``: every head divided by its root mean square after rotation; ``value_mix``: 1 keeps the
+    values in ``v_first``, 2 blends them with it by the device scalar ``mix``."""
+    n, ld = proj.shape
+    nkv, hdp = cache.n_kv_heads, cache.head_dim
+    dt = cache.pool.dtype
+    half = rotated_dims // 2
+    call("fl_qkv_prepare", _check(proj, "qkv_prepare.proj", torch.float32), ld, *(int(c) for c in cols),
+         _check(positions, "qkv_prepare.positions", torch.int32, (n,)), _check(tok_seq, "qkv_prepare.tok_seq", torch.int32, (n,)),
+         _check(block_table, "qkv_prepare.block_table", torch.int32, (None, None)), block_table.shape[1],
+         _check(q_out, "qkv_prepare.q_out", dt, (n, n_heads * hdp)), _check(cache.pool, "qkv_prepare.cache"), dtype_code(dt),
+         n, int(n_heads), nkv, int(dim), int(vdim), hdp, cache.page_size, cache.n_pages, int(rotated_dims), int(bool(interleaved)),
+         _check(table, "qkv_prepare.table", torch.float32, (n, half, 2)) if rotated_dims else None,
+         _check(q_gain, "qkv_prepare.q_gain", torch.float32, (n_heads * dim,)) if q_gain is not None else None,
+         _check(k_gain, "qkv_prepare.k_gain", torch.float32, (nkv * dim,)) if k_gain is not None else None,
+         int(bool(head_norm)), float(eps),
+         _check(v_first, "qkv_prepare.v_first", torch.float32, (n, nkv * vdim)) if v_first is not None else None, int(value_mix),
+         _check(mix, "qkv_prepare.mix", torch.float32) if mix is not None else None, int(bool(write_cache)), stream_handle())
+    return q_out
+
+
+def linear_scan_max_dim() -> int:
+    from .library import load
+    return load().fl_linear_scan_max_dim()
+
+
+def conv_max_taps() -> int:
+    from .library import load
+    return load().fl_conv_max_taps()
+
+
+def linear_scan(q, k, v, state, seq_q_start, seq_q_len, seq_slots, out, n_heads, n_qk_heads, dim, vdim,
+                head_decay=None, token_gates=None):
+    """The recurrence S <- g S + k u^T, o = S^T q over the step's tokens, request by request, from and into
+    the first ``heads * dim * vdim`` floats of every slot's record in ``state`` ``[slots, floats]``.
+    ``q``, ``k`` float32 ``[n, n_qk_heads * dim]`` (views of wider rows are taken with their row stride),
+    ``v`` ``[n, n_heads * vdim]``.  ``head_decay`` float32 ``[heads]``: a fixed g per head and u = v;
+    ``token_gates`` float32 ``[n, 2 * heads]`` (g, then beta): the delta rule, u = beta (v - S^T k)."""
+    n = out.shape[0]
+    S = seq_q_start.shape[0]
+    if state.dim() != 2 or not state.is_contiguous():
+        raise KernelError(f"linear_scan.state: shape {tuple(state.shape)}, expected [slots, floats]")
+
+    def rows(t, name, width):
+        if t.dtype != torch.float32 or not t.is_cuda or t.dim() != 2 or t.shape != (n, width) or t.stride(1) != 1:
+            raise KernelError(f"linear_scan.{name}: {t.dtype} {tuple(t.shape)}, want float32 [{n}, {width}] with unit stride")
+        return t.data_ptr(), t.stride(0)
+    (pq, ldq), (pk, ldk), (pv, ldv) = rows(q, "q", n_qk_heads * dim), rows(k, "k", n_qk_heads * dim), rows(v, "v", n_heads * vdim)
+    if (head_decay is None) == (token_gates is None):
+        raise KernelError("linear_scan: a decay per head or gates per token, one of the two")
+    pg = _check(token_gates, "linear_scan.gates", torch.float32, (n, 2 * n_heads)) if token_gates is not None else None
+    call("fl_linear_scan", pq, ldq, pk, ldk, pv, ldv,
+         _check(head_decay, "linear_scan.decay", torch.float32, (n_heads,)) if head_decay is not None else None,
+         pg, pg + 4 * n_heads if pg is not None else None, 2 * n_heads if pg is not None else 0,
+         _check(state, "linear_scan.state", torch.float32), state.shape[1],
+         _check(seq_q_start, "linear_scan.seq_q_start", torch.int32, (S,)), _check(seq_q_len, "linear_scan.seq_q_len", torch.int32, (S,)),
+         _check(seq_slots, "linear_scan.seq_slots", torch.int32, (S,)), _check(out, "linear_scan.out", torch.float32, (n, n_heads * vdim)),
+         S, int(n_heads), int(n_qk_heads), int(dim), int(vdim), stream_handle())
+    return out
+
+
+def conv_prepare(proj, col0, col_b, col_a, conv_w, a_log, dt_bias, state, conv_at, tok_seq, seq_q_start, seq_q_len, seq_slots,
+                 prep, gates, n_qk_heads, n_heads, dim, vdim, taps, q_scale, unit_eps):
+    """Short causal convolution + silu over the channels of q, k, v (columns ``col0`` on of the float32 rows
+    ``proj``), unit vectors per head of q (times ``q_scale``) and k, and the gates of every (token, head) into
+    ``gates`` ``[n, 2 * heads]`` (decay, then write strength).  The inputs of the last ``taps - 1`` tokens of a
+    request live at ``conv_at`` floats into its record of ``state`` ``[slots, floats]`` and are moved on."""
+    n, ld = proj.shape
+    S = seq_q_start.shape[0]
+    C = 2 * n_qk_heads * dim + n_heads * vdim
+    if state.dim() != 2 or not state.is_contiguous() or state.shape[1] < conv_at + (taps - 1) * C:
+        raise KernelError(f"conv_prepare.state: shape {tuple(state.shape)} does not hold {taps - 1} x {C} floats at {conv_at}")
+    call("fl_conv_prepare", _check(proj, "conv_prepare.proj", torch.float32), ld, int(col0), int(col_b), int(col_a),
+         _check(conv_w, "conv_prepare.conv_w", torch.float32, (C, taps)), _check(a_log, "conv_prepare.a_log", torch.float32, (n_heads,)),
+         _check(dt_bias, "conv_prepare.dt_bias", torch.float32, (n_heads,)),
+         _check(state, "conv_prepare.state", torch.float32) + 4 * int(conv_at), state.shape[1],
+         _check(tok_seq, "conv_prepare.tok_seq", torch.int32, (n,)), _check(seq_q_start, "conv_prepare.seq_q_start", torch.int32, (S,)),
+         _check(seq_q_len, "conv_prepare.seq_q_len", torch.int32, (S,)), _check(seq_slots, "conv_prepare.seq_slots", torch.int32, (S,)),
+         _check(prep, "conv_prepare.prep", torch.float32, (n, C)), _check(gates, "conv_prepare.gates", torch.float32, (n, 2 * n_heads)),
+         n, S, int(n_qk_heads), int(n_heads), int(dim), int(vdim), int(taps), float(q_scale), float(unit_eps), stream_handle())
+    return prep
+
+
+def rotate_scale(proj, col_a, col_b, table, rotated_dims, interleaved, scale_a, scale_b, out_a, out_b, n_heads, dim):
+    """Two sets of heads in the float32 rows ``proj`` (at ``col_a`` and ``col_b``) rotated by the step's table
+    and multiplied by a factor each, into float32 ``out_a`` and ``out_b`` ``[n, heads * dim]``."""
+    n, ld = proj.shape
+    call("fl_rotate_scale", _check(proj, "rotate_scale.proj", torch.float32), ld, int(col_a), int(col_b),
+         _check(table, "rotate_scale.table", torch.float32, (n, rotated_dims // 2, 2)) if rotated_dims else None,
+         int(rotated_dims), int(bool(interleaved)), float(scale_a), float(scale_b),
+         _check(out_a, "rotate_scale.out_a", torch.float32, (n, n_heads * dim)),
+         _check(out_b, "rotate_scale.out_b", torch.float32, (n, n_heads * dim)), n, int(n_heads), int(dim), stream_handle())

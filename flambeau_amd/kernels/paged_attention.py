@@ -26,9 +26,10 @@ class PlainPagedAttention:
         product and rotation apart."""
         return False
 
-    def attention(self, q, out, kv, step, table, n_heads: int, scale: float, window: int):
-        """Grouped-query attention of the step's rows over the paged cache."""
-        return ops.attn_plain(q, out, kv, step.positions, step.tok_seq, table, n_heads, scale, window)
+    def attention(self, q, out, kv, step, table, n_heads: int, scale: float, window: int, softcap: float = 0.0):
+        """Grouped-query attention of the step's rows over the paged cache; ``softcap`` > 0 caps the
+        scores, ``softcap * tanh(score / softcap)``, before the softmax."""
+        return ops.attn_plain(q, out, kv, step.positions, step.tok_seq, table, n_heads, scale, window, softcap=softcap)
 
     def metadata(self, batch, mixers) -> dict:
         """Integer arrays the kernels want uploaded with the step (work lists); none here."""
@@ -51,9 +52,9 @@ class TunedPagedAttention(PlainPagedAttention):
         store = tuned.RopeStore(step.positions, step.tok_seq, table, angles, q_out, kv, n_heads, rotated_dims, writes)
         return tuned.gemm_rope_store(x, w, store, rt=self.rt)
 
-    def attention(self, q, out, kv, step, table, n_heads, scale, window):
+    def attention(self, q, out, kv, step, table, n_heads, scale, window, softcap=0.0):
         from . import tuned
-        return tuned.attention(self.rt, q, out, kv, step, table, n_heads, scale, window)
+        return tuned.attention(self.rt, q, out, kv, step, table, n_heads, scale, window, softcap=softcap)
 
     def metadata(self, batch, mixers):
         """The rows and tiles of the batch, and for the single-row kernel the rows with splits of their

@@ -45,6 +45,8 @@ register_signatures({
     "fl_attn_prefill_takes": [I, I, I, I],
     "fl_attn_decode": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, P],
     "fl_attn_decode_items": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, P, I, P],
+    "fl_attn_decode_items_capped": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, F, P, I, P],
+    "fl_attn_prefill_capped": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, F, I, P, P, I, P],
 })
 
 SKINNY_MAX_ROWS = 64     # rows the decode kernels take
@@ -668,7 +670,8 @@ def decode_splits(n_items: int, n_kv_heads: int, group: int, max_ctx: int) -> in
     return int(min(by_blocks, by_keys, 64))
 
 
-def attn_decode(q, out, cache, rows, table, n_heads, scale, window, n_split, part_o=None, part_ml=None, firsts=None):
+def attn_decode(q, out, cache, rows, table, n_heads, scale, window, n_split, part_o=None, part_ml=None, firsts=None,
+                softcap: float = 0.0):
     """Attention of single query rows; ``rows[i] = (row of q and out, position, index of the request's
     row in ``table``, 0)``, every row's keys in ``n_split`` parts; or, with ``n_split`` = 0, rows with
     splits of their own as ``balanced_items`` lists them, with its list ``firsts`` of where each row's
@@ -687,7 +690,13 @@ def attn_decode(q, out, cache, rows, table, n_heads, scale, window, n_split, par
             _check(cache.pool, "attn.cache", torch.bfloat16), _check(rows, "attn.rows", torch.int32, (n_items, 4)), n_items,
             _check(table, "attn.block_table", torch.int32, (None, None)), table.shape[1], n_heads, cache.n_kv_heads,
             hd, cache.page_size, cache.n_pages, float(scale), int(window))
-    if n_split == 0:
+    if softcap and n_split != 0:
+        raise KernelError("attn_decode: capped scores come with rows that have splits of their own (n_split = 0)")
+    if n_split == 0 and softcap:
+        call("fl_attn_decode_items_capped", *head, float(softcap),
+             _check(firsts, "attn.firsts", torch.int32, (None, 4)) if firsts is not None else None,
+             firsts.shape[0] if firsts is not None else 0, stream_handle())
+    elif n_split == 0:
         call("fl_attn_decode_items", *head, _check(firsts, "attn.firsts", torch.int32, (None, 4)) if firsts is not None else None,
              firsts.shape[0] if firsts is not None else 0, stream_handle())
     else:
@@ -710,7 +719,7 @@ def attn_prefill_heads(n_tiles: int, n_heads: int, n_kv_heads: int, head_dim: in
 
 
 def attn_prefill(q, out, cache, tiles, positions, table, n_heads, scale, window, heads_per_wave: int = 0,
-                 n_split: int = 1, part_o=None, part_ml=None):
+                 n_split: int = 1, part_o=None, part_ml=None, softcap: float = 0.0):
     """Attention of the longer portions; ``tiles[i] = (request's row in ``table``, first row, rows,
     index of the first row among all rows of tiles)``.  With ``n_split`` > 1 the keys are split and
     merged; ``part_o`` / ``part_ml``: float32 workspaces of rows x heads x n_split x (head_dim rounded
@@ -725,12 +734,12 @@ def attn_prefill(q, out, cache, tiles, positions, table, n_heads, scale, window,
             raise KernelError("attn_prefill: splits need a workspace")
         if n_rows is not None and (part_o.numel() < n_rows * n_heads * n_split * hdp or part_ml.numel() < n_rows * n_heads * n_split * 2):
             raise KernelError("attn_prefill: workspace too small for the splits")
-    call("fl_attn_prefill", _check(q, "attn.q", torch.bfloat16, (n, n_heads * hd)),
+    call("fl_attn_prefill_capped" if softcap else "fl_attn_prefill", _check(q, "attn.q", torch.bfloat16, (n, n_heads * hd)),
          _check(out, "attn.out", torch.bfloat16, (n, n_heads * hd)), _check(cache.pool, "attn.cache", torch.bfloat16),
          _check(tiles, "attn.tiles", torch.int32, (n_tiles, 4)), n_tiles,
          _check(positions, "attn.positions", torch.int32, (n,)),
          _check(table, "attn.block_table", torch.int32, (None, None)), table.shape[1], n_heads, cache.n_kv_heads, hd,
-         cache.page_size, cache.n_pages, float(scale), int(window), int(heads_per_wave),
+         cache.page_size, cache.n_pages, float(scale), int(window), *((float(softcap),) if softcap else ()), int(heads_per_wave),
          _check(part_o, "attn.part_o", torch.float32) if part_o is not None else None,
          _check(part_ml, "attn.part_ml", torch.float32) if part_ml is not None else None, int(n_split), stream_handle())
     return out
@@ -781,15 +790,16 @@ def attention_splits(batch, n_heads: int, n_kv_heads: int, head_dim: int, window
     return p_split, n_split
 
 
-def attention(rt, q, out, cache, step, table, n_heads, scale, window):
+def attention(rt, q, out, cache, step, table, n_heads, scale, window, softcap: float = 0.0):
     """Attention of one batch with the tuned kernels: rows of short portions through the split-K
     kernel, longer portions through the tiled kernel.  A cache shape one of them does not take
     sends the whole batch to the plain kernel."""
     rows, tiles = step.extra.get("attn_rows"), step.extra.get("attn_tiles")
     batch = step.host
-    if rows is None or tiles is None or not decode_supported(cache) or (tiles.shape[0] and not prefill_supported(cache, table, window)):
-        return ops.attn_plain(q, out, cache, step.positions, step.tok_seq, table, n_heads, scale, window)
-    items = step.extra.get(f"attn_items/{decode_blocks_per_row(n_heads, cache.n_kv_heads)}/{window or 0}")
+    items = step.extra.get(f"attn_items/{decode_blocks_per_row(n_heads, cache.n_kv_heads)}/{window or 0}") if rows is not None else None
+    if rows is None or tiles is None or not decode_supported(cache) or (tiles.shape[0] and not prefill_supported(cache, table, window)) \
+            or (softcap and items is None):
+        return ops.attn_plain(q, out, cache, step.positions, step.tok_seq, table, n_heads, scale, window, softcap=softcap)
     key = ("attention_splits", n_heads, cache.n_kv_heads, cache.head_dim, window)
     splits = step.scratch.get(key)
     if splits is None:
@@ -805,7 +815,7 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
             p_o = rt.buffer("attn_tile_part_o", n_rows * n_heads * p_split, hdp, torch.float32, max_rows=1 << 24)
             p_ml = rt.buffer("attn_tile_part_ml", n_rows * n_heads * p_split, 2, torch.float32, max_rows=1 << 24)
         attn_prefill(q, out, cache, tiles, step.positions, table, n_heads, scale, window, heads_per_wave=p_heads,
-                     n_split=p_split, part_o=p_o, part_ml=p_ml)
+                     n_split=p_split, part_o=p_o, part_ml=p_ml, softcap=softcap)
     if rows.shape[0] and items is not None:
         # rows with splits of their own; the list's length follows from the number of rows alone
         # (a list with a place per row and no more: no row is ever split, nothing to merge)
@@ -818,7 +828,7 @@ def attention(rt, q, out, cache, step, table, n_heads, scale, window):
             slots = items.shape[0] * n_heads
             part_o = rt.buffer("attn_part_o", slots, hdp, torch.float32, max_rows=1 << 24)
             part_ml = rt.buffer("attn_part_ml", slots, 2, torch.float32, max_rows=1 << 24)
-        attn_decode(q, out, cache, items, table, n_heads, scale, window, 0, part_o, part_ml, firsts=firsts)
+        attn_decode(q, out, cache, items, table, n_heads, scale, window, 0, part_o, part_ml, firsts=firsts, softcap=softcap)
     elif rows.shape[0]:
         part_o = part_ml = None
         if n_split > 1:

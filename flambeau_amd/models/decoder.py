@@ -147,6 +147,19 @@ class DecoderModel:
             todo += list(getattr(p, "subparts", lambda: [])())
         return True
 
+    @staticmethod
+    def _mixers_of(block) -> list:
+        """A block's mixers, and the mixers inside a mixer that is made of several (``Mixer.mixers``)."""
+        out, todo = [], list(getattr(block, "mixers", lambda: [])())
+        while todo:
+            m = todo.pop(0)
+            inner = list(getattr(m, "mixers", lambda: [])())
+            if inner:
+                todo = inner + todo
+            else:
+                out.append(m)
+        return out
+
     def step_signature(self, batch) -> tuple:
         """What the mixers decide from the batch's numbers beyond its shape (``Mixer.step_signature``),
         one entry per group of like mixers.  Mixers of blocks that are never recorded decide anew in
@@ -156,7 +169,7 @@ class DecoderModel:
             for b in self.blocks:
                 if not self._part_replayable(b):
                     continue
-                for m in getattr(b, "mixers", lambda: [])():
+                for m in self._mixers_of(b):
                     seen.setdefault(m.signature_group(), m)
             self._signature_mixers = list(seen.values())
         return tuple(m.step_signature(batch) for m in self._signature_mixers)
@@ -168,7 +181,7 @@ class DecoderModel:
         """The model's mixers, grouped by their class in the order of first appearance."""
         found = {}
         for b in self.blocks:
-            for m in getattr(b, "mixers", lambda: [])():
+            for m in self._mixers_of(b):
                 found.setdefault(type(m), []).append(m)
         return found
 

@@ -105,3 +105,117 @@ class PagedGQAAttention(Mixer):
         out = rt.buffer("attn_out", n, nh * hd)
         self.kernels.attention(q, out, cache.kv, step, table, nh, self.scale, self.window)
         return Product(out, self.w_o)
+
+
+@MIXERS.register("normed_gqa_attention")
+class NormedGQAAttention(PagedGQAAttention):
+    """Grouped-query attention over the paged cache with the extras of newer designs, each a parameter:
+
+    * ``value_dim``: values of another size than queries and keys.  The cache keeps heads
+      ``max(head_dim, value_dim)`` wide (rounded up to 8), keys and values padded with zeros, so that the
+      attention kernels of one head size serve both;
+    * ``qk_norm``: ``"projection"``: q (and k) divided by the root mean square over ALL its heads at once,
+      times a gain per value, before rotation; ``"head"``: every head of q and k divided by its own root
+      mean square after rotation, no gain; ``None``;
+    * ``position``: any encoding that offers a table of cosines and sines and a ``layout`` (``half`` or
+      ``interleaved``), or ``none``;
+    * ``softcap``: score <- softcap * tanh(score / softcap) before the softmax;
+    * ``value_mix``: ``"source"``: this layer's values are kept for later layers of the step;
+      ``"blend"``: v <- (1 - lambda) v + lambda v_source with a learned lambda, and the blend is what
+      the cache holds.  Both read and write ``StepState.scratch[value_mix_key]``;
+    * ``gate``: the heads' outputs times ``sigmoid`` (or ``silu``) of a projection of the mixer's input,
+      value by value, before the output projection.
+
+    One joined product gives q, k, v and the gate's logits in 32-bit; norms, rotation and the blend are
+    32-bit; this step's keys are stored before attention runs."""
+    graph_safe = True
+    lazy_input = False
+    replayable = True
+
+    def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PartSpec,
+                 value_dim: int | None = None, window: int = 0, scale: float | None = None, qk_norm: str | None = None,
+                 eps: float = 1e-6, softcap: float | None = None, value_mix: str | None = None,
+                 value_mix_key: str = "value_mix", gate: str | None = None):
+        value_dim = head_dim if value_dim is None else value_dim
+        self.value_dim = value_dim
+        self.stored_dim = -(-max(head_dim, value_dim) // 8) * 8
+        if qk_norm not in (None, "projection", "head"):
+            raise ValueError(f"normed_gqa_attention: qk_norm must be 'projection', 'head' or None, got {qk_norm!r}")
+        if value_mix not in (None, "source", "blend"):
+            raise ValueError(f"normed_gqa_attention: value_mix must be 'source', 'blend' or None, got {value_mix!r}")
+        if gate not in ops.HEAD_GATES:
+            raise ValueError(f"normed_gqa_attention: gate must be 'sigmoid', 'silu' or None, got {gate!r}")
+        super().__init__(hidden_size, n_heads, n_kv_heads, self.stored_dim, position, window, scale)
+        self.head_dim = head_dim                      # (the base class checked the stored size against the kernels)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.qk_norm, self.eps = qk_norm, float(eps)
+        self.softcap = float(softcap or 0.0)
+        self.value_mix, self.value_mix_key, self.gate = value_mix, value_mix_key, gate
+
+    def cache_spec(self):
+        return PagedKVSpec(self.n_kv_heads, self.stored_dim, self.window)
+
+    def signature_group(self):
+        return ("normed_gqa_attention", self.n_heads, self.n_kv_heads, self.stored_dim, self.window)
+
+    def step_signature(self, batch):
+        return self.kernels.signature(batch, self.n_heads, self.n_kv_heads, self.stored_dim, self.window)
+
+    def tensors(self):
+        W, H, G, D, Dv = self.hidden_size, self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim
+        t = {"q.weight": TensorSpec((H * D, W)), "k.weight": TensorSpec((G * D, W)), "v.weight": TensorSpec((G * Dv, W)),
+             "o.weight": TensorSpec((W, H * Dv))}
+        if self.qk_norm == "projection":
+            t["q_norm.weight"] = TensorSpec((H * D,), "vector32")
+            t["k_norm.weight"] = TensorSpec((G * D,), "vector32")
+        if self.value_mix is not None:
+            # (the layer whose values are the source has the scalar too, and does not use it)
+            t["value_mix.weight"] = TensorSpec((), "vector32", init=lambda g, shape, device: torch.rand(shape, generator=g, device=device))
+        if self.gate is not None:
+            t["g.weight"] = TensorSpec((H * Dv, W))
+        return t
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.kernels = rt.kernels("paged_attention")
+        H, G, D, Dv = self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim
+        joined = [weights["q.weight"], weights["k.weight"], weights["v.weight"]] + ([weights["g.weight"]] if self.gate else [])
+        self.w_in = rt.prepare_weight(torch.cat(joined, dim=0).contiguous())
+        self.cols = (0, H * D, H * D + G * D)
+        self.gate_col = H * D + G * D + G * Dv
+        self.q_gain, self.k_gain = weights.get("q_norm.weight"), weights.get("k_norm.weight")
+        self.mix = weights["value_mix.weight"].reshape(1) if self.value_mix == "blend" else None
+        self.w_o = rt.prepare_weight(weights["o.weight"])
+        self.position.bind({}, rt)
+        self.rotated_dims = int(getattr(self.position, "rotated_dims", 0) or 0)      # (the encoding 'none' has none)
+        self.interleaved = getattr(self.position, "layout", "half") == "interleaved"
+        if self.rotated_dims and not hasattr(self.position, "rotary_table"):
+            raise ValueError("normed_gqa_attention: the position encoding offers no table of cosines and sines")
+
+    def forward(self, x, step, cache):
+        rt, n = self.rt, x.shape[0]
+        H, G, D, Dv, P = self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim, self.stored_dim
+        table = step.block_tables[cache.group]
+        proj = rt.buffer("nattn_proj", n, self.w_in.rows, torch.float32)
+        rt.gemm(x, self.w_in, proj)
+        angles = self.position.rotary_table(rt, step) if self.rotated_dims else None
+        v_first, mode = None, 0
+        if self.value_mix == "source":
+            v_first = step.scratch[self.value_mix_key] = rt.buffer("nattn_" + self.value_mix_key, n, G * Dv, torch.float32)
+            mode = 1
+        elif self.value_mix == "blend":
+            v_first = step.scratch.get(self.value_mix_key)
+            if v_first is None or v_first.shape != (n, G * Dv):
+                raise RuntimeError("normed_gqa_attention: no layer before this one has left values of this shape to blend with")
+            mode = 2
+        q = rt.buffer("nattn_q", n, H * P)
+        ops.qkv_prepare(proj, self.cols, step.positions, step.tok_seq, table, q, cache.kv, H, D, Dv, self.rotated_dims,
+                        self.interleaved, angles, self.q_gain, self.k_gain, self.qk_norm == "head", self.eps,
+                        v_first=v_first, value_mix=mode, mix=self.mix, write_cache=cache.writes)
+        out = rt.buffer("nattn_out", n, H * P)
+        self.kernels.attention(q, out, cache.kv, step, table, H, self.scale, self.window, softcap=self.softcap)
+        if self.gate is not None or P != Dv:
+            gated = rt.buffer("nattn_gated", n, H * Dv)
+            ops.heads_gate(out, P, proj if self.gate is not None else None, self.gate_col, self.gate, gated, H)
+            out = gated
+        return Product(out, self.w_o)

@@ -142,6 +142,45 @@ class StateSpec(CacheSpec):
         return torch.zeros((max_slots, *self.shape), dtype=self.dtype, device=device)
 
 
+@dataclass(frozen=True)
+class JoinedCacheSpec(CacheSpec):
+    """The caches of a mixer made of several: at most one of them paged, the records per slot of the others
+    side by side in one record (``state_offsets`` says where each begins, in values of ``dtype``)."""
+    paged: CacheSpec | None
+    states: tuple                  # of StateSpec (or None for a member without one)
+
+    def page_group(self):
+        return self.paged.page_group() if self.paged is not None else None
+
+    def allocate_pool(self, n_entries, n_pages, page_size, dtype, device):
+        return self.paged.allocate_pool(n_entries, n_pages, page_size, dtype, device)
+
+    def layer_view(self, pool, index):
+        return self.paged.layer_view(pool, index)
+
+    def state_offsets(self):
+        out, at = [], 0
+        for s in self.states:
+            out.append(at)
+            if s is not None:
+                n = 1
+                for d in s.shape:
+                    n *= d
+                at += n
+        return out, at
+
+    def allocate_state(self, max_slots, device):
+        kinds = {s.dtype for s in self.states if s is not None}
+        if not kinds:
+            return None
+        if len(kinds) > 1:
+            raise ValueError("the per-slot records of a joined cache must share a dtype")
+        return torch.zeros((max_slots, self.state_offsets()[1]), dtype=kinds.pop(), device=device)
+
+    def bytes_per_token(self, element_size):
+        return self.paged.bytes_per_token(element_size) if self.paged is not None else 0
+
+
 @dataclass
 class LayerCache:
     """What one run-order entry sees of the cache."""

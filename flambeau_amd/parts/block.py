@@ -57,13 +57,16 @@ class ResidualStream:
 class PreNormBlock(Block):
     replayable = True
 
-    def __init__(self, mixer: PartSpec, feed_forward: PartSpec, norm: PartSpec):
+    def __init__(self, mixer: PartSpec, feed_forward: PartSpec | None, norm: PartSpec):
+        """``feed_forward`` may be ``None``: a layer of a mixer alone, x += Mixer(Norm1(x)), with no second norm."""
         self.mixer_norm = NORMS.create(norm)
         self.mixer = MIXERS.create(mixer)
-        self.ffn_norm = NORMS.create(norm)
-        self.ffn = FEED_FORWARDS.create(feed_forward)
-        self._parts = {"mixer_norm": self.mixer_norm, "mixer": self.mixer,
-                       "ffn_norm": self.ffn_norm, "ffn": self.ffn}
+        self._parts = {"mixer_norm": self.mixer_norm, "mixer": self.mixer}
+        self.ffn = None
+        if feed_forward is not None:
+            self.ffn_norm = NORMS.create(norm)
+            self.ffn = FEED_FORWARDS.create(feed_forward)
+            self._parts.update({"ffn_norm": self.ffn_norm, "ffn": self.ffn})
 
     def cache_spec(self):
         return self.mixer.cache_spec()
@@ -84,7 +87,8 @@ class PreNormBlock(Block):
 
     def forward(self, stream, step, cache):
         stream.push(self.mixer.forward(stream.normed(self.mixer_norm, lazy=self.mixer.lazy_input), step, cache))
-        stream.push(self.ffn.forward(stream.normed(self.ffn_norm, lazy=self.ffn.lazy_input), step))
+        if self.ffn is not None:
+            stream.push(self.ffn.forward(stream.normed(self.ffn_norm, lazy=self.ffn.lazy_input), step))
 
 
 @BLOCKS.register("parallel")

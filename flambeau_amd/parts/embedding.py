@@ -59,3 +59,15 @@ class OutputHead(Part):
         logits = self.rt.buffer("logits", x.shape[0], self.vocab_size, torch.float32, max_rows=max_rows)
         self.rt.gemm(x, self.weight, logits)
         return logits
+
+
+@EMBEDDINGS.register("scaled_token_embedding")
+class ScaledTokenEmbedding(TokenEmbedding):
+    """h0[i, :] = E[token[i], :] * scale, the product taken in 32-bit."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float):
+        super().__init__(vocab_size, hidden_size)
+        self.scale = float(scale)
+
+    def forward(self, tokens, out):
+        return ops.embed_scaled(self.weight, tokens, out, self.scale)

@@ -30,3 +30,33 @@ class RMSNorm(Norm):
         leaves the norm in factors: x * w in the compute dtype and the sums of squares in parts.
         The product that follows multiplies by rsqrt(mean + eps) itself: no norm kernel runs."""
         return rt.gemm_add_norm(product.x, product.weight, resid, self.weight, self.eps)
+
+
+@NORMS.register("dynamic_tanh")
+class DynamicTanh(Norm):
+    """y = tanh(alpha x) * w + b: a norm that takes no mean and no variance, so nothing crosses the values
+    of a row.  ``alpha`` is one learned number, ``w`` and ``b`` vectors; ``bias=False`` leaves b out."""
+    replayable = True
+
+    def __init__(self, hidden_size: int, bias: bool = True, alpha_init: float = 0.5):
+        self.hidden_size = hidden_size
+        self.has_bias = bool(bias)
+        self.alpha_init = float(alpha_init)
+
+    def tensors(self):
+        import torch
+        a0 = self.alpha_init
+        t = {"weight": TensorSpec((self.hidden_size,), "vector32"),
+             "alpha": TensorSpec((), "vector32", init=lambda g, shape, device: torch.full(shape, a0, device=device) * (
+                 1.0 + 0.1 * torch.randn(shape, generator=g, device=device)))}
+        if self.has_bias:
+            t["bias"] = TensorSpec((self.hidden_size,), "vector32", init="normal")
+        return t
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.weight, self.alpha = weights["weight"], weights["alpha"].reshape(1)
+        self.bias = weights.get("bias")
+
+    def forward(self, x, out, delta=None, store_sum=False, rows=None):
+        return ops.dyt(x, self.alpha, self.weight, self.bias, out, delta=delta, store_sum=store_sum, rows=rows)

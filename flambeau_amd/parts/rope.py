@@ -74,3 +74,52 @@ class NoPositionEncoding(PositionEncoding):
 
     def rotary_parameters(self):
         return 0, 1.0
+
+
+@POSITION_ENCODINGS.register("rope_interleaved")
+class RotaryInterleaved(RotaryNeoX):
+    """The same angles with the other pairing: dimension 2i turns with dimension 2i + 1.  The fused
+    rotate-and-store kernels pair split halves, so this encoding offers its table and its ``layout``
+    to mixers whose kernels read both."""
+    layout = "interleaved"
+
+    def rotary_parameters(self):
+        return None
+
+
+RotaryNeoX.layout = "half"
+
+
+def blended_frequencies(rotated_dims: int, theta: float, factor: float, original: int, fast: float, slow: float):
+    """A ladder of frequencies stretched for contexts beyond ``original`` positions: a dimension whose wave
+    makes fewer than ``slow`` turns over ``original`` positions has its frequency divided by ``factor``, one
+    that makes more than ``fast`` turns keeps it, and those between are mixed linearly in the dimension's
+    index.  With ``turn(n) = dims * ln(original / (2 pi n)) / (2 ln theta)`` the (fractional) index whose
+    wave makes n turns: lo = max(floor(turn(fast)), 0), hi = min(ceil(turn(slow)), dims - 1),
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), f_i' = f_i / factor * ramp_i + f_i (1 - ramp_i).
+    Returns the frequencies and the factor 0.1 ln(factor) + 1 that goes on every cosine and sine."""
+    import math
+    def turn(n):
+        return rotated_dims * math.log(original / (2.0 * math.pi * n)) / (2.0 * math.log(theta))
+    lo = max(math.floor(turn(fast)), 0)
+    hi = min(math.ceil(turn(slow)), rotated_dims - 1)
+    out = []
+    for i in range(rotated_dims // 2):
+        f = theta ** (-2.0 * i / rotated_dims)
+        ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+        out.append(f / factor * ramp + f * (1.0 - ramp))
+    return out, 0.1 * math.log(factor) + 1.0
+
+
+@POSITION_ENCODINGS.register("rope_blended")
+class RotaryBlended(RotaryNeoX):
+    """Split-half rotation with the stretched ladder of ``blended_frequencies``."""
+
+    def __init__(self, head_dim: int, theta: float, factor: float, original: int, fast: float, slow: float,
+                 rotated_dims: int | None = None):
+        super().__init__(head_dim, theta, rotated_dims)
+        self._freqs, self.magnitude = blended_frequencies(self.rotated_dims, self.theta, float(factor), int(original),
+                                                           float(fast), float(slow))
+
+    def inverse_frequencies(self):
+        return self._freqs
