@@ -130,7 +130,8 @@ def rotated_attention(h, t, p, m, eps):
     k = (h @ t[p + "k"].T).reshape(T, G, D)
     v = (h @ t[p + "v"].T).reshape(T, G, Dv)
     pos = np.arange(T)
-    q, k = rotate(q, pos, m["rot"], "half"), rotate(k, pos, m["rot"], "half")
+    if m.get("rot"):
+        q, k = rotate(q, pos, m["rot"], "half"), rotate(k, pos, m["rot"], "half")
     q, k = rms_norm(q, None, eps), rms_norm(k, None, eps)
     o = causal_softmax_attention(q, k, v, m["scale"])
     return o.reshape(T, H * Dv) @ t[p + "o"].T
@@ -145,7 +146,9 @@ def retention(h, t, p, m, eps):
     k = (h @ t[p + "k"].T).reshape(T, H, D)
     v = (h @ t[p + "v"].T).reshape(T, H, Dv)
     pos = np.arange(T)
-    q, k = rotate(q, pos, m["rot"], "half"), rotate(k, pos, m["rot"], "half") * D ** -0.5
+    if m.get("rot"):
+        q, k = rotate(q, pos, m["rot"], "half"), rotate(k, pos, m["rot"], "half")
+    k = k * D ** -0.5
     o = np.zeros((T, H, Dv))
     for a in range(H):
         S = np.zeros((D, Dv))
@@ -167,8 +170,8 @@ def short_convolution(x, w):
     """x [T, C], w [C, taps]: y[i] = sum_j w[:, taps - 1 - j] x[i - j], zeros before the start."""
     T, taps = x.shape[0], w.shape[1]
     y = np.zeros_like(x)
-    for j in range(taps):
-        y[j:] += x[:T - j] * w[:, taps - 1 - j] if j else x * w[:, taps - 1]
+    for j in range(min(taps, T)):
+        y[j:] += x[:T - j] * w[:, taps - 1 - j]
     return y
 
 
