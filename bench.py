@@ -21,6 +21,10 @@ and Mistral-Nemo-12B sizes, 64 requests with prompts of 128 to 4,096 tokens and 
 stretch) at two sizes that resemble real layers, random weights, beside a Mistral of the same width, head count and
 number of layer runs: a 2,048-token prompt as one step and decode steps of 8 requests behind 2,048 tokens each.  One
 JSON line; ``value`` is Kuvidra's decode tokens/s at the larger size, the rest is under ``points``.
+
+``--config bugidra``: the Bugidra design (attention with normed, capped and gated extras, attention and retention side
+by side, the gated delta rule behind short convolutions, Dynamic Tanh norms) at two sizes that resemble real layers,
+beside a Mistral of the same width, head count and number of layers, measured the same way; a line of the same shape.
 """
 from __future__ import annotations
 
@@ -371,20 +375,49 @@ KUVIDRA_SIZES = {
 }
 
 
+def bugidra_config(width, heads, kv_heads, ff, ret_heads, delta_heads, delta_qk_heads, vocab=32768):
+    att = {"type": "attention", "mixer": dict(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=128 ** -0.5, softcap=50.0, v_mix=True,
+                                              rot={"base": 10000.0, "dims": 64})}
+    left = dict(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=0.09,
+                rot={"base": 50000.0, "dims": 128, "scaling": {"factor": 2.0, "original": 4096, "fast": 32.0, "slow": 1.0}})
+    right = dict(heads=ret_heads, dim=128, vdim=128, decay=[1.0 - 2.0 ** -(5 + i % 8) for i in range(ret_heads)],
+                 rot={"base": 1e6, "dims": 128})
+    par = {"type": "parallel", "mixer": {"left": left, "right": right}}
+    delta = {"type": "delta", "mixer": dict(heads=delta_heads, kv_heads=delta_qk_heads, dim=128, vdim=128, conv=4)}
+    mlp = {"kind": "dense", "ff": ff}
+    return {"architecture": "Bugidra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": width ** 0.5},
+            "layers": [dict(l, mlp=mlp) for l in (delta, par, att, delta, par, att)]}
+
+
+BUGIDRA_SIZES = {
+    "w2048": dict(width=2048, heads=16, kv_heads=8, ff=8192, ret_heads=8, delta_heads=16, delta_qk_heads=8),
+    "w4096": dict(width=4096, heads=32, kv_heads=8, ff=14336, ret_heads=16, delta_heads=32, delta_qk_heads=16),
+}
+
+
 def bench_kuvidra(a, dtype_name):
     """Prefill and decode of the Kuvidra design at layer sizes of real models, beside the closest model the engine
     has (Mistral) at the same width, head count and number of layer runs."""
+    return bench_design(a, dtype_name, "kuvidra", "Kuvidra", KUVIDRA_SIZES, kuvidra_config, "6 layer runs")
+
+
+def bench_bugidra(a, dtype_name):
+    """The same for the Bugidra design: six layers (two of each kind) beside a Mistral of six layers."""
+    return bench_design(a, dtype_name, "bugidra", "Bugidra", BUGIDRA_SIZES, bugidra_config, "6 layers")
+
+
+def bench_design(a, dtype_name, design, title, all_sizes, make_config, runs_text):
     import torch
     from flambeau_amd import random_model
     points = {}
-    for name, sz in KUVIDRA_SIZES.items():
+    for name, sz in all_sizes.items():
         if a.only_size and a.only_size != name:
             continue
-        kcfg = kuvidra_config(**sz)
-        runs = 6           # four layers, two of them twice
+        kcfg = make_config(**sz)
+        runs = 6           # layer runs of either design's configuration
         mcfg = dict(_BASE, num_hidden_layers=runs, hidden_size=sz["width"], num_attention_heads=sz["heads"], num_key_value_heads=8,
                     head_dim=128, intermediate_size=sz["ff"], vocab_size=32768, rope_theta=1e6, sliding_window=None)
-        for label, cfg in (("kuvidra", kcfg), ("mistral", mcfg)):
+        for label, cfg in ((design, kcfg), ("mistral", mcfg)):
             if a.only_model and a.only_model != label:
                 continue
             model, _ = random_model(cfg, seed=0, dtype=dtype_name, max_batch_tokens=PROMPT_LEN + 64, std=0.02, gain_std=0.0)
@@ -400,12 +433,12 @@ def bench_kuvidra(a, dtype_name):
                     points[f"{key}_decode_b{b}_ms"] = round(dt * 1e3, 3)
             del model
             torch.cuda.empty_cache()
-    head = points.get("w4096_kuvidra_decode_b8_tok_s")
-    out = {"metric": f"decode tok/s (Kuvidra design, width 4096, 6 layer runs, {a.dtype}, batch 8 behind 2,048 tokens)",
+    head = points.get(f"w4096_{design}_decode_b8_tok_s")
+    out = {"metric": f"decode tok/s ({title} design, width 4096, {runs_text}, {a.dtype}, batch 8 behind 2,048 tokens)",
            "value": head, "unit": "tokens/s", "n_gpus": 1, "steps": 24, "warmup": 6,
-           "ms_per_step": points.get("w4096_kuvidra_decode_b8_ms"), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "ms_per_step": points.get(f"w4096_{design}_decode_b8_ms"), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": a.dtype, "data": "synthetic: random weights N(0, 0.02^2), uniform random token ids, caches filled with random values for decode",
-           "config": {"model": "Kuvidra design at two sizes beside Mistral of equal width", "sizes": KUVIDRA_SIZES,
+           "config": {"model": f"{title} design at two sizes beside Mistral of equal width", "sizes": all_sizes,
                       "global_batch": 8, "seq_len": PROMPT_LEN, "parallelism": "single GPU"},
            "points": points}
     print(json.dumps(out), flush=True)
@@ -419,9 +452,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--reps", type=int, default=REPS, help="repetitions of the timed steps; the median is reported")
-    ap.add_argument("--config", default="7b", choices=sorted(CONFIGS) + ["kuvidra"])
-    ap.add_argument("--only-size", default=None, choices=sorted(KUVIDRA_SIZES), help="--config kuvidra: one size only")
-    ap.add_argument("--only-model", default=None, choices=["kuvidra", "mistral"], help="--config kuvidra: one of the two models only")
+    ap.add_argument("--config", default="7b", choices=sorted(CONFIGS) + ["kuvidra", "bugidra"])
+    ap.add_argument("--only-size", default=None, choices=sorted(KUVIDRA_SIZES), help="--config kuvidra / bugidra: one size only")
+    ap.add_argument("--only-model", default=None, choices=["kuvidra", "bugidra", "mistral"],
+                    help="--config kuvidra / bugidra: one of the two models only")
     ap.add_argument("--layers", type=int, default=None, help="run only the first layers (named in config)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
@@ -438,6 +472,8 @@ def main():
     el = 2 if a.dtype == "bf16" else 4
     if a.config == "kuvidra":
         return bench_kuvidra(a, dtype_name)
+    if a.config == "bugidra":
+        return bench_bugidra(a, dtype_name)
     label, cfg = CONFIGS[a.config]
     if a.config != "7b":
         return bench_serving(a, a.config, label, cfg, dtype_name, el)

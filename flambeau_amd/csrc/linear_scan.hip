@@ -27,15 +27,23 @@
 #define LS_COLS 16           // columns of S per block
 #define LS_MAX_ROWS 32       // rows per thread: D <= LS_GROUP * LS_MAX_ROWS
 #define LS_MAX_TAPS 16
+#define LS_QK_REGS 8          // values of a q or k head per lane in the kernel that prepares them: D <= 512
 
 // Block = (columns j0 .. j0 + 15, head, request); thread (g, c) holds S[d][j0 + c] for its rows d.
 // State of a head: S column by column, S[d][j] at j * D + d.
+// The step's tokens come through LDS a run of RUN tokens at a time; the next run's values are asked for
+// (into registers) before the walk over this run begins and put into LDS after it, so that the trip to
+// memory hides behind the walk.
 template <int RPT, bool DELTA>
 __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
     const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk, const float* __restrict__ v, int ldv,
     const float* __restrict__ head_decay, const float* __restrict__ tok_decay, const float* __restrict__ beta, int ldg,
     float* __restrict__ state, size_t slot_stride, const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
-    const int* __restrict__ seq_slots, float* __restrict__ out, int H, int G, int D, int Dv, int run) {
+    const int* __restrict__ seq_slots, float* __restrict__ out, int H, int G, int D, int Dv) {
+    constexpr int NT = LS_GROUP * LS_COLS;
+    constexpr int RUN = RPT <= 8 ? 32 : RPT <= 16 ? 16 : 8;          // tokens per run: RUN * (2 D + 18) floats of LDS
+    constexpr int PRE = RUN * LS_GROUP * RPT / NT;                    // q (and k) values of a run per thread
+    constexpr int PRE_V = (RUN * LS_COLS + NT - 1) / NT;
     const int g = threadIdx.x & (LS_GROUP - 1), c = threadIdx.x / LS_GROUP;
     const int j = blockIdx.x * LS_COLS + c, head = blockIdx.y, s = blockIdx.z;
     const int qk_head = head / (H / G);
@@ -49,29 +57,46 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
         S[u] = (live && d < D) ? st[(size_t)j * D + d] : 0.f;
     }
     const float fixed = head_decay ? head_decay[head] : 1.f;
-    // the step's tokens come through LDS a run at a time: one trip to memory per run, not one per token
-    extern __shared__ float ls_smem[];
-    float* qs = ls_smem;                          // [run][D]
-    float* ks = qs + (size_t)run * D;             // [run][D]
-    float* vs = ks + (size_t)run * D;             // [run][16]
-    float* fs = vs + (size_t)run * LS_COLS;       // [run][2]: decay, beta
-    for (int t0 = 0; t0 < len; t0 += run) {
-        const int cnt = min(run, len - t0);
-        __syncthreads();
-        for (int e = threadIdx.x; e < cnt * D; e += LS_GROUP * LS_COLS) {
+    __shared__ float qs[RUN * LS_GROUP * RPT], ks[RUN * LS_GROUP * RPT], vs[RUN * LS_COLS], fs[RUN * 2];
+    float pq[PRE], pk[PRE], pv[PRE_V], pf0 = 0.f, pf1 = 0.f;
+    auto fetch = [&](int t0) {                     // the values of the run that starts at token t0, into registers
+        const int cnt = min(RUN, len - t0);
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            const int e = threadIdx.x + NT * i;
             const int tt = e / D, d = e - tt * D;
-            qs[e] = q[(size_t)(start + t0 + tt) * ldq + qk_head * D + d];
-            ks[e] = k[(size_t)(start + t0 + tt) * ldk + qk_head * D + d];
+            const bool in = tt < cnt;
+            const size_t row = (size_t)(start + t0 + (in ? tt : 0));
+            pq[i] = in ? q[row * ldq + qk_head * D + d] : 0.f;
+            pk[i] = in ? k[row * ldk + qk_head * D + d] : 0.f;
         }
-        for (int e = threadIdx.x; e < cnt * LS_COLS; e += LS_GROUP * LS_COLS) {
+#pragma unroll
+        for (int i = 0; i < PRE_V; ++i) {
+            const int e = threadIdx.x + NT * i;
             const int tt = e / LS_COLS, jj = blockIdx.x * LS_COLS + (e - tt * LS_COLS);
-            vs[e] = jj < Dv ? v[(size_t)(start + t0 + tt) * ldv + head * Dv + jj] : 0.f;
+            pv[i] = (tt < cnt && jj < Dv) ? v[(size_t)(start + t0 + tt) * ldv + head * Dv + jj] : 0.f;
         }
-        for (int tt = threadIdx.x; tt < cnt; tt += LS_GROUP * LS_COLS) {
-            fs[2 * tt] = tok_decay ? tok_decay[(size_t)(start + t0 + tt) * ldg + head] : fixed;
-            fs[2 * tt + 1] = DELTA ? beta[(size_t)(start + t0 + tt) * ldg + head] : 1.f;
+        if (threadIdx.x < cnt) {
+            const size_t row = (size_t)(start + t0 + threadIdx.x);
+            pf0 = tok_decay ? tok_decay[row * ldg + head] : fixed;
+            pf1 = DELTA ? beta[row * ldg + head] : 1.f;
         }
+    };
+    if (len > 0) fetch(0);
+    for (int t0 = 0; t0 < len; t0 += RUN) {
+        const int cnt = min(RUN, len - t0);
+        __syncthreads();                           // the walk over the run before has read its last value
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            const int e = threadIdx.x + NT * i;
+            if (e < RUN * D) { qs[e] = pq[i]; ks[e] = pk[i]; }
+        }
+#pragma unroll
+        for (int i = 0; i < PRE_V; ++i)
+            if (threadIdx.x + NT * i < RUN * LS_COLS) vs[threadIdx.x + NT * i] = pv[i];
+        if (threadIdx.x < RUN) { fs[2 * threadIdx.x] = pf0; fs[2 * threadIdx.x + 1] = pf1; }
         __syncthreads();
+        if (t0 + RUN < len) fetch(t0 + RUN);
         for (int tt = 0; tt < cnt; ++tt) {
             const float decay = fs[2 * tt];
             float uv = vs[tt * LS_COLS + c];
@@ -122,13 +147,10 @@ extern "C" int fl_linear_scan(const float* q, int ldq, const float* k, int ldk, 
     FL_CHECK(n_seqs <= 65535 && H <= 65535, "linear_scan: %d requests of %d heads are more than one grid takes", n_seqs, H);
     dim3 grid(ceil_div(Dv, LS_COLS), H, n_seqs);
     const int rpt = ceil_div(D, LS_GROUP);
-    int run = (60 * 1024) / ((2 * D + LS_COLS + 2) * (int)sizeof(float));
-    run = run > 32 ? 32 : (run < 1 ? 1 : run);
-    const size_t lds = (size_t)run * (2 * D + LS_COLS + 2) * sizeof(float);
 #define FL_LS2(R, DELTA)                                                                                              \
-    linear_scan_kernel<R, DELTA><<<grid, LS_GROUP * LS_COLS, lds, stream>>>(q, ldq, k, ldk, v, ldv, head_decay, tok_decay, beta, \
-                                                                            ldg, state, (size_t)slot_stride, seq_q_start,        \
-                                                                            seq_q_len, seq_slots, out, H, G, D, Dv, run)
+    linear_scan_kernel<R, DELTA><<<grid, LS_GROUP * LS_COLS, 0, stream>>>(q, ldq, k, ldk, v, ldv, head_decay, tok_decay, beta, \
+                                                                          ldg, state, (size_t)slot_stride, seq_q_start,        \
+                                                                          seq_q_len, seq_slots, out, H, G, D, Dv)
 #define FL_LS(R)             \
     do {                     \
         if (beta) FL_LS2(R, true); \
@@ -159,6 +181,8 @@ struct ConvPrepare {
     float q_scale, unit_eps;
 };
 
+// A wave per (token, head of q, k or v): a lane takes the head's channels lane, lane + 64, ...; the heads of a
+// token are spread over blocks of four waves, so that a step of few tokens still fills units.
 __global__ __launch_bounds__(256) void conv_prepare_kernel(ConvPrepare a) {
     const int token = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int C = 2 * a.G * a.D + a.H * a.Dv, taps = a.taps;
@@ -166,16 +190,7 @@ __global__ __launch_bounds__(256) void conv_prepare_kernel(ConvPrepare a) {
     const int back = token - a.seq_q_start[s];            // tokens of the request in this step before this one
     const float* hist = a.conv_state + (size_t)a.seq_slots[s] * a.slot_stride;
     float* dst = a.prep + (size_t)token * C;
-    for (int c = threadIdx.x; c < C; c += 256) {
-        float y = 0.f;
-        for (int jj = taps - 1; jj >= 0; --jj) {          // oldest input first
-            const float x = jj <= back ? a.proj[(size_t)(token - jj) * a.ld + a.col0 + c]
-                                       : hist[(size_t)(taps - 1 - (jj - back)) * C + c];
-            y = fmaf(a.conv_w[(size_t)c * taps + (taps - 1 - jj)], x, y);
-        }
-        dst[c] = y / (1.0f + expf(-y));
-    }
-    if (threadIdx.x < a.H) {
+    if (blockIdx.y == 0 && threadIdx.x < a.H) {
         const int h = threadIdx.x;
         const float* row = a.proj + (size_t)token * a.ld;
         const float z = row[a.col_a + h] + a.dt_bias[h];
@@ -183,15 +198,37 @@ __global__ __launch_bounds__(256) void conv_prepare_kernel(ConvPrepare a) {
         a.gates[(size_t)token * 2 * a.H + h] = expf(-expf(a.a_log[h]) * sp);
         a.gates[(size_t)token * 2 * a.H + a.H + h] = 1.0f / (1.0f + expf(-row[a.col_b + h]));
     }
-    __syncthreads();
-    // q heads, then k heads: unit vectors
-    for (int head = wave; head < 2 * a.G; head += 4) {
-        float* x = dst + (size_t)head * a.D;
-        float ss = 0.f;
-        for (int d = lane; d < a.D; d += 64) ss = fmaf(x[d], x[d], ss);
-        const float f = (head < a.G ? a.q_scale : 1.f) / sqrtf(wave_sum(ss) + a.unit_eps);
-        for (int d = lane; d < a.D; d += 64) x[d] *= f;
+    const int unit = blockIdx.y * 4 + wave;
+    if (unit >= 2 * a.G + a.H) return;
+    const bool is_qk = unit < 2 * a.G;
+    const int width = is_qk ? a.D : a.Dv;
+    const int c0 = is_qk ? unit * a.D : 2 * a.G * a.D + (unit - 2 * a.G) * a.Dv;
+    auto convolved = [&](int c) {
+        float y = 0.f;
+        for (int jj = taps - 1; jj >= 0; --jj) {          // oldest input first
+            const float x = jj <= back ? a.proj[(size_t)(token - jj) * a.ld + a.col0 + c]
+                                       : hist[(size_t)(taps - 1 - (jj - back)) * C + c];
+            y = fmaf(a.conv_w[(size_t)c * taps + (taps - 1 - jj)], x, y);
+        }
+        return y / (1.0f + expf(-y));
+    };
+    if (!is_qk) {
+        for (int d = lane; d < width; d += 64) dst[c0 + d] = convolved(c0 + d);
+        return;
     }
+    // q and k heads become unit vectors (D <= 64 * LS_QK_REGS, checked on the host)
+    float r[LS_QK_REGS];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < LS_QK_REGS; ++j) {
+        const int d = lane + 64 * j;
+        r[j] = d < width ? convolved(c0 + d) : 0.f;
+        ss = fmaf(r[j], r[j], ss);
+    }
+    const float f = (unit < a.G ? a.q_scale : 1.f) / sqrtf(wave_sum(ss) + a.unit_eps);
+#pragma unroll
+    for (int j = 0; j < LS_QK_REGS; ++j)
+        if (lane + 64 * j < width) dst[c0 + lane + 64 * j] = r[j] * f;
 }
 
 // per (request, channel): the kept inputs move on by the request's tokens of this step
@@ -233,7 +270,10 @@ extern "C" int fl_conv_prepare(const float* proj, int ld, int col0, int col_b, i
     FL_CHECK(n_seqs <= 65535, "conv_prepare: %d requests are more than one grid takes", n_seqs);
     ConvPrepare a{proj, ld, col0, col_b, col_a, conv_w, a_log, dt_bias, conv_state, (size_t)slot_stride, tok_seq, seq_q_start,
                   seq_slots, prep, gates, G, H, D, Dv, taps, q_scale, unit_eps};
-    conv_prepare_kernel<<<n, 256, 0, stream>>>(a);
+    FL_CHECK(D <= 64 * LS_QK_REGS, "conv_prepare: %d key dims per head, at most %d", D, 64 * LS_QK_REGS);
+    dim3 pgrid(n, ceil_div(2 * G + H, 4));
+    FL_CHECK(pgrid.y <= 65535, "conv_prepare: %d heads are more than one grid takes", 2 * G + H);
+    conv_prepare_kernel<<<pgrid, 256, 0, stream>>>(a);
     FL_LAUNCH_CHECK();
     if (taps > 1 && n_seqs > 0) {
         dim3 grid(ceil_div(C, 256), n_seqs);

@@ -47,8 +47,10 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __res
         prow = pos % cache.page_size;
     }
     const int half = a.rot >> 1;
-    // q and k heads: a wave per head, a lane per head dim (and the dims 64, 128, ... further)
-    for (int head = wave; head < nh + nkv; head += 4) {
+    // q and k heads: a wave per head, a lane per head dim (and the dims 64, 128, ... further); the heads of a token
+    // are spread over blocks of four waves (every block forms the projection's sums of squares for itself)
+    const int head = blockIdx.y * 4 + wave;
+    if (head < nh + nkv) {
         const bool is_q = head < nh;
         const int h = is_q ? head : head - nh;
         const float* src = row + (is_q ? a.col_q : a.col_k) + h * D;
@@ -92,9 +94,9 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __res
                 if (lane + 64 * j < hdp) dst[lane + 64 * j] = from_f32<T>(r[j]);
         }
     }
-    // v heads
+    // v heads: the blocks share their values out
     const float lam = a.vmix_mode == 2 ? a.lambda[0] : 0.f;
-    for (int e = threadIdx.x; e < nkv * hdp; e += 256) {
+    for (int e = blockIdx.y * 256 + threadIdx.x; e < nkv * hdp; e += 256 * gridDim.y) {
         const int h = e / hdp, d = e - h * hdp;
         float v = 0.f;
         if (d < Dv) {
@@ -125,10 +127,12 @@ extern "C" int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, i
     QkvPrepare a{proj, ld, col_q, col_k, col_v, positions, tok_seq, block_table, max_blocks, nh, D, Dv, hdp,
                  rot, interleaved, (const float2*)cs, qnorm_w, knorm_w, head_norm, eps, v_first, vmix_mode, lambda, write_cache};
     PagedCache c{cache_base, nkv, page_size, hdp, n_pages};
+    dim3 grid(n, ceil_div(nh + nkv, 4));
+    FL_CHECK(grid.y <= 65535, "qkv_prepare: %d heads are more than one grid takes", nh + nkv);
     if (dtype == FL_F32)
-        qkv_prepare_kernel<float><<<n, 256, 0, stream>>>(a, (float*)q_out, c);
+        qkv_prepare_kernel<float><<<grid, 256, 0, stream>>>(a, (float*)q_out, c);
     else if (dtype == FL_BF16)
-        qkv_prepare_kernel<bf16_t><<<n, 256, 0, stream>>>(a, (bf16_t*)q_out, c);
+        qkv_prepare_kernel<bf16_t><<<grid, 256, 0, stream>>>(a, (bf16_t*)q_out, c);
     else
         FL_CHECK(false, "qkv_prepare: unknown dtype %d", dtype);
     FL_LAUNCH_CHECK();

@@ -9,6 +9,8 @@
 // ------------------------------------------------------------------ Dynamic Tanh
 // out[r][i] = tanh(alpha * s) * w[i] + b[i], s = x[row][i] (+ delta[row][i]); with resid_out the sum is
 // written back.  No mean, no variance: nothing crosses the elements of a row.
+// A thread takes four neighbouring values of a row (one 16-byte load where the width allows it); a row is
+// spread over as many blocks as it has thousands of values, so that a step of few rows still fills units.
 template <typename TOut>
 __global__ __launch_bounds__(256) void dyt_kernel(const float* __restrict__ x, const float* __restrict__ delta,
                                                   float* __restrict__ resid_out, const int* __restrict__ rows,
@@ -17,11 +19,29 @@ __global__ __launch_bounds__(256) void dyt_kernel(const float* __restrict__ x, c
     const int r = blockIdx.x;
     const size_t row = rows ? (size_t)rows[r] : (size_t)r;
     const float a = alpha[0];
-    for (int i = threadIdx.x; i < H; i += 256) {
-        float s = x[row * H + i];
-        if (delta) s += delta[row * H + i];
-        if (resid_out) resid_out[row * H + i] = s;
-        out[(size_t)r * H + i] = from_f32<TOut>(tanhf(a * s) * w[i] + (b ? b[i] : 0.f));
+    const int i0 = (blockIdx.y * 256 + threadIdx.x) * 4;
+    if (i0 >= H) return;
+    float s[4];
+    if ((H & 3) == 0) {
+        const f32x4 v = *(const f32x4*)(x + row * H + i0);
+        s[0] = v[0]; s[1] = v[1]; s[2] = v[2]; s[3] = v[3];
+        if (delta) {
+            const f32x4 d = *(const f32x4*)(delta + row * H + i0);
+            s[0] += d[0]; s[1] += d[1]; s[2] += d[2]; s[3] += d[3];
+        }
+        if (resid_out) *(f32x4*)(resid_out + row * H + i0) = (f32x4){s[0], s[1], s[2], s[3]};
+    } else {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = i0 + u;
+            s[u] = i < H ? x[row * H + i] + (delta ? delta[row * H + i] : 0.f) : 0.f;
+            if (resid_out && i < H) resid_out[row * H + i] = s[u];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u;
+        if (i < H) out[(size_t)r * H + i] = from_f32<TOut>(tanhf(a * s[u]) * w[i] + (b ? b[i] : 0.f));
     }
 }
 
@@ -31,10 +51,12 @@ extern "C" int fl_dyt(const float* x, const float* delta, float* resid_out, cons
     FL_CHECK(alpha && w, "dyt: needs alpha and a gain");
     FL_CHECK(!(rows && resid_out), "dyt: picked rows are not stored back");
     if (n_rows == 0) return 0;
+    FL_CHECK(ceil_div(H, 1024) <= 65535, "dyt: rows of %d values are more than one grid takes", H);
+    dim3 grid(n_rows, ceil_div(H, 1024));
     if (out_dtype == FL_F32)
-        dyt_kernel<float><<<n_rows, 256, 0, stream>>>(x, delta, resid_out, rows, alpha, w, b, (float*)out, H);
+        dyt_kernel<float><<<grid, 256, 0, stream>>>(x, delta, resid_out, rows, alpha, w, b, (float*)out, H);
     else if (out_dtype == FL_BF16)
-        dyt_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(x, delta, resid_out, rows, alpha, w, b, (bf16_t*)out, H);
+        dyt_kernel<bf16_t><<<grid, 256, 0, stream>>>(x, delta, resid_out, rows, alpha, w, b, (bf16_t*)out, H);
     else
         FL_CHECK(false, "dyt: unknown dtype %d", out_dtype);
     FL_LAUNCH_CHECK();
@@ -79,17 +101,27 @@ __device__ __forceinline__ float activate(float z, int kind) {
 template <typename TOut>
 __global__ __launch_bounds__(256) void gated_act_kernel(const float* __restrict__ gu, TOut* __restrict__ out, int I, int kind) {
     const float* row = gu + (size_t)blockIdx.x * 2 * I;
-    for (int i = threadIdx.x; i < I; i += 256) out[(size_t)blockIdx.x * I + i] = from_f32<TOut>(activate(row[i], kind) * row[I + i]);
+    const int i0 = (blockIdx.y * 256 + threadIdx.x) * 4;        // four neighbouring values per thread, a row over several blocks
+    if (i0 >= I) return;
+    if ((I & 3) == 0) {
+        const f32x4 g = *(const f32x4*)(row + i0), u = *(const f32x4*)(row + I + i0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[(size_t)blockIdx.x * I + i0 + e] = from_f32<TOut>(activate(g[e], kind) * u[e]);
+    } else {
+        for (int i = i0; i < min(i0 + 4, I); ++i) out[(size_t)blockIdx.x * I + i] = from_f32<TOut>(activate(row[i], kind) * row[I + i]);
+    }
 }
 
 extern "C" int fl_gated_act(const float* gu, void* out, int out_dtype, int n, int I, int kind, hipStream_t stream) {
     FL_CHECK(n >= 0 && I > 0, "gated_act: bad sizes");
     FL_CHECK(kind >= 0 && kind <= 2, "gated_act: unknown activation %d", kind);
     if (n == 0) return 0;
+    FL_CHECK(ceil_div(I, 1024) <= 65535, "gated_act: rows of %d values are more than one grid takes", I);
+    dim3 grid(n, ceil_div(I, 1024));
     if (out_dtype == FL_F32)
-        gated_act_kernel<float><<<n, 256, 0, stream>>>(gu, (float*)out, I, kind);
+        gated_act_kernel<float><<<grid, 256, 0, stream>>>(gu, (float*)out, I, kind);
     else if (out_dtype == FL_BF16)
-        gated_act_kernel<bf16_t><<<n, 256, 0, stream>>>(gu, (bf16_t*)out, I, kind);
+        gated_act_kernel<bf16_t><<<grid, 256, 0, stream>>>(gu, (bf16_t*)out, I, kind);
     else
         FL_CHECK(false, "gated_act: unknown dtype %d", out_dtype);
     FL_LAUNCH_CHECK();
