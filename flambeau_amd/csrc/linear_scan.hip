@@ -29,11 +29,12 @@
 #define LS_MAX_TAPS 16
 #define LS_QK_REGS 8          // values of a q or k head per lane in the kernel that prepares them: D <= 512
 
-// Block = (columns j0 .. j0 + 15, head, request); thread (g, c) holds S[d][j0 + c] for its rows d.
+// Block = (columns j0 .. j0 + 15, head, request); thread (g, c) holds S[d][j0 + c] for its RPT rows
+// d = g * RPT .. g * RPT + RPT - 1 (neighbours, so that its q and k come from LDS in 16-byte reads).
 // State of a head: S column by column, S[d][j] at j * D + d.
-// The step's tokens come through LDS a run of RUN tokens at a time; the next run's values are asked for
-// (into registers) before the walk over this run begins and put into LDS after it, so that the trip to
-// memory hides behind the walk.
+// The step's tokens come through LDS a run of RUN tokens at a time, rows 16 * RPT wide and zero behind D;
+// the next run's values are asked for (into registers) before the walk over this run begins and put into
+// LDS after it, so that the trip to memory hides behind the walk.
 template <int RPT, bool DELTA>
 __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
     const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk, const float* __restrict__ v, int ldv,
@@ -41,8 +42,9 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
     float* __restrict__ state, size_t slot_stride, const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
     const int* __restrict__ seq_slots, float* __restrict__ out, int H, int G, int D, int Dv) {
     constexpr int NT = LS_GROUP * LS_COLS;
-    constexpr int RUN = RPT <= 8 ? 32 : RPT <= 16 ? 16 : 8;          // tokens per run: RUN * (2 D + 18) floats of LDS
-    constexpr int PRE = RUN * LS_GROUP * RPT / NT;                    // q (and k) values of a run per thread
+    constexpr int DP = LS_GROUP * RPT;                                // a row of q or k in LDS
+    constexpr int RUN = RPT <= 8 ? 32 : RPT <= 16 ? 16 : 8;          // tokens per run
+    constexpr int PRE = RUN * DP / NT;                                // q (and k) values of a run per thread
     constexpr int PRE_V = (RUN * LS_COLS + NT - 1) / NT;
     const int g = threadIdx.x & (LS_GROUP - 1), c = threadIdx.x / LS_GROUP;
     const int j = blockIdx.x * LS_COLS + c, head = blockIdx.y, s = blockIdx.z;
@@ -53,19 +55,21 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
     float S[RPT];
 #pragma unroll
     for (int u = 0; u < RPT; ++u) {
-        const int d = g + LS_GROUP * u;
+        const int d = g * RPT + u;
         S[u] = (live && d < D) ? st[(size_t)j * D + d] : 0.f;
     }
     const float fixed = head_decay ? head_decay[head] : 1.f;
-    __shared__ float qs[RUN * LS_GROUP * RPT], ks[RUN * LS_GROUP * RPT], vs[RUN * LS_COLS], fs[RUN * 2];
+    __shared__ __attribute__((aligned(16))) float qs[RUN * DP];
+    __shared__ __attribute__((aligned(16))) float ks[RUN * DP];
+    __shared__ float vs[RUN * LS_COLS], fs[RUN * 2];
     float pq[PRE], pk[PRE], pv[PRE_V], pf0 = 0.f, pf1 = 0.f;
     auto fetch = [&](int t0) {                     // the values of the run that starts at token t0, into registers
         const int cnt = min(RUN, len - t0);
 #pragma unroll
         for (int i = 0; i < PRE; ++i) {
             const int e = threadIdx.x + NT * i;
-            const int tt = e / D, d = e - tt * D;
-            const bool in = tt < cnt;
+            const int tt = e / DP, d = e % DP;
+            const bool in = tt < cnt && d < D;
             const size_t row = (size_t)(start + t0 + (in ? tt : 0));
             pq[i] = in ? q[row * ldq + qk_head * D + d] : 0.f;
             pk[i] = in ? k[row * ldk + qk_head * D + d] : 0.f;
@@ -88,8 +92,8 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
         __syncthreads();                           // the walk over the run before has read its last value
 #pragma unroll
         for (int i = 0; i < PRE; ++i) {
-            const int e = threadIdx.x + NT * i;
-            if (e < RUN * D) { qs[e] = pq[i]; ks[e] = pk[i]; }
+            qs[threadIdx.x + NT * i] = pq[i];
+            ks[threadIdx.x + NT * i] = pk[i];
         }
 #pragma unroll
         for (int i = 0; i < PRE_V; ++i)
@@ -97,36 +101,43 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
         if (threadIdx.x < RUN) { fs[2 * threadIdx.x] = pf0; fs[2 * threadIdx.x + 1] = pf1; }
         __syncthreads();
         if (t0 + RUN < len) fetch(t0 + RUN);
+#pragma unroll 2
         for (int tt = 0; tt < cnt; ++tt) {
             const float decay = fs[2 * tt];
             float uv = vs[tt * LS_COLS + c];
-            float kr[RPT];
+            float kr[RPT], qr[RPT];
 #pragma unroll
             for (int u = 0; u < RPT; ++u) {
-                const int d = g + LS_GROUP * u;
-                kr[u] = d < D ? ks[tt * D + d] : 0.f;
+                kr[u] = ks[tt * DP + g * RPT + u];
+                qr[u] = qs[tt * DP + g * RPT + u];
                 S[u] *= decay;
             }
             if (DELTA) {
-                float seen = 0.f;
+                float seen0 = 0.f, seen1 = 0.f;                   // two chains of half the length
 #pragma unroll
-                for (int u = 0; u < RPT; ++u) seen = fmaf(S[u], kr[u], seen);
-                uv = fs[2 * tt + 1] * (uv - row_sum16(seen));
+                for (int u = 0; u < RPT; u += 2) {
+                    seen0 = fmaf(S[u], kr[u], seen0);
+                    if (u + 1 < RPT) seen1 = fmaf(S[u + 1], kr[u + 1], seen1);
+                }
+                uv = fs[2 * tt + 1] * (uv - row_sum16(seen0 + seen1));
             }
-            float num = 0.f;
+            float num0 = 0.f, num1 = 0.f;
 #pragma unroll
-            for (int u = 0; u < RPT; ++u) {
-                const int d = g + LS_GROUP * u;
+            for (int u = 0; u < RPT; u += 2) {
                 S[u] = fmaf(kr[u], uv, S[u]);
-                num = fmaf(S[u], d < D ? qs[tt * D + d] : 0.f, num);
+                num0 = fmaf(S[u], qr[u], num0);
+                if (u + 1 < RPT) {
+                    S[u + 1] = fmaf(kr[u + 1], uv, S[u + 1]);
+                    num1 = fmaf(S[u + 1], qr[u + 1], num1);
+                }
             }
-            num = row_sum16(num);                                  // the 16 threads of a column are a row of lanes
+            const float num = row_sum16(num0 + num1);             // the 16 threads of a column are a row of lanes
             if (live && g == 0) out[((size_t)(start + t0 + tt) * H + head) * Dv + j] = num;
         }
     }
 #pragma unroll
     for (int u = 0; u < RPT; ++u) {
-        const int d = g + LS_GROUP * u;
+        const int d = g * RPT + u;
         if (live && d < D) st[(size_t)j * D + d] = S[u];
     }
 }
