@@ -38,6 +38,17 @@ template <typename T> __device__ __forceinline__ T from_f32(float v);
 template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return (bf16_t)v; }
 
+// The gate of a gated feed-forward, act(gate) * up: 0 silu, 1 gelu in its tanh form, 2 gelu with the error function.
+// (The codes that launch functions take in the bits of `epilogue` above the low four.)
+#define FL_GATE_SILU 0
+#define FL_GATE_GELU_TANH 1
+#define FL_GATE_GELU_ERF 2
+__device__ __forceinline__ float gate_activation(float z, int kind) {
+    if (kind == FL_GATE_GELU_TANH) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+    if (kind == FL_GATE_GELU_ERF) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+    return z / (1.0f + expf(-z));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, FL_WAVE);

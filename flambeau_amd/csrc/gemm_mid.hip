@@ -47,7 +47,7 @@ template <> __device__ __forceinline__ void gm_store4<bf16_t>(bf16_t* p, f32x4 v
 template <int MT, int GM_NW, int GM_CH, typename TOut, bool SWIGLU>
 __global__ __launch_bounds__(GM_NW * 64) void gemm_mid_kernel(const bf16_t* x, const bf16_t* wp, TOut* out, int M, int N, int K,
                                                               int n_steps, int chunks_per_split, int out_cols,
-                                                              const float* in_ssq, int in_parts, float eps) {
+                                                              const float* in_ssq, int in_parts, float eps, int gate_kind) {
     constexpr int FR = GM_CH * MT;                    // 1 KB operand tiles of x per chunk
     constexpr int XL = (FR + GM_NW - 1) / GM_NW;      // x loads per wave and chunk
     __shared__ __attribute__((aligned(16))) bf16_t slots[2][FR * 512];
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(GM_NW * 64) void gemm_mid_kernel(const bf16_t* x, c
             if ((g & 1) == 0 && tok < M && f0 < out_cols) {
                 f32x4 act;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) act[r] = acc[mt][r] / (1.0f + expf(-acc[mt][r])) * up[r];
+                for (int r = 0; r < 4; ++r) act[r] = gate_activation(acc[mt][r], gate_kind) * up[r];
                 TOut* p = out + (size_t)tok * out_cols + f0;
                 if (out_cols % 4 == 0 && f0 + 4 <= out_cols) {
                     gm_store4<TOut>(p, act);
@@ -354,6 +354,7 @@ struct MidScale {              // the row scale of a product whose x is a norm i
     const float* in_ssq;
     int in_parts;
     float eps;
+    int gate_kind;             // the SwiGLU epilogue's activation of the gate (FL_GATE_*, 0 = silu)
 };
 
 template <int MT, int NW, int CH, typename TOut, bool SWIGLU>
@@ -364,7 +365,7 @@ static void launch_mid_shape(const bf16_t* x, const bf16_t* wp, TOut* out, int M
     const int per = ceil_div(n_chunks, splits);
     dim3 grid(ceil_div(ceil_div(N, 16), NW), splits);
     gemm_mid_kernel<MT, NW, CH, TOut, SWIGLU><<<grid, NW * 64, 0, stream>>>(x, wp, out, M, N, K, n_steps, per, out_cols,
-                                                                            sc.in_ssq, sc.in_parts, sc.eps);
+                                                                            sc.in_ssq, sc.in_parts, sc.eps, sc.gate_kind);
 }
 
 template <int MT, typename TOut, bool SWIGLU>
@@ -405,7 +406,10 @@ extern "C" int fl_gemm_mid_ex(const void* x, const void* w_packed, void* out, fl
     FL_CHECK(waves == 0 || waves == 4 || waves == 8, "gemm_mid: %d waves per block (0, 4 or 8)", waves);
     if (mid_checks(x, w_packed, M, N, K)) return -1;
     FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_mid: unknown output dtype %d", out_dtype);
+    const int gate_kind = epilogue >> 4;          // the bits above the low four: the activation of the gate (epilogue 1)
+    epilogue &= 15;
     FL_CHECK(epilogue == 0 || epilogue == 1, "gemm_mid: unknown epilogue %d", epilogue);
+    FL_CHECK(gate_kind >= 0 && gate_kind <= FL_GATE_GELU_ERF && (gate_kind == 0 || epilogue == 1), "gemm_mid: gate activation %d", gate_kind);
     FL_CHECK(epilogue == 0 ? out_cols == N : (N % 16 == 0 && out_cols > 0 && out_cols <= N / 2),
              "gemm_mid: %d output columns do not fit %d rows of w", out_cols, N);
     FL_CHECK((uintptr_t)out % 16 == 0, "gemm_mid: operands must be 16-byte aligned");
@@ -416,7 +420,7 @@ extern "C" int fl_gemm_mid_ex(const void* x, const void* w_packed, void* out, fl
     const int mt = ceil_div(M, 16);
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w_packed;
-    const MidScale sc = {in_ssq, in_parts, eps};
+    const MidScale sc = {in_ssq, in_parts, eps, gate_kind};
     const MidPlan plan = epilogue ? MidPlan{mid_waves(N, waves), 1} : mid_plan(N, K, waves, forced_splits);
     const int splits = plan.splits;
     waves = plan.waves;

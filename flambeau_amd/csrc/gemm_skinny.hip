@@ -53,6 +53,7 @@ struct SkinnyFusion {
     const float* g;           // epilogue 2: [N] weight of the following norm
     bf16_t* xg;               // epilogue 2: [M][N] bf16(resid * g)
     float* out_ssq;           // epilogue 2: [M][blocks] sum of resid^2 over the block's features
+    int gate_kind;            // epilogue 1: the gate's activation (FL_GATE_*, 0 = silu)
 };
 
 #define SKINNY_SCALE_LOADS 4     // loads of partial sums per thread for the row scale
@@ -317,7 +318,7 @@ __global__ __launch_bounds__(T == 1 ? 1024 : 512) void gemm_skinny_kernel(const 
                 if ((g & 1) == 0 && tok < M && f0 < out_cols) {
                     f32x4 act;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) act[r] = sum[r] / (1.0f + expf(-sum[r])) * up[r];
+                    for (int r = 0; r < 4; ++r) act[r] = gate_activation(sum[r], fu.gate_kind) * up[r];
                     TOut* p = out + (size_t)tok * out_cols + f0;
                     if (out_cols % 4 == 0 && f0 + 4 <= out_cols) {
                         store4(p, act);
@@ -434,8 +435,14 @@ static int launch_skinny(const bf16_t* x, const bf16_t* wp, TOut* out, int M, in
 }
 
 static int skinny_entry(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N, int K,
-                        int nw_hint, int epilogue, int out_cols, const SkinnyFusion& fu, const RopeStore& rs,
+                        int nw_hint, int epilogue, int out_cols, const SkinnyFusion& fusion, const RopeStore& rs,
                         hipStream_t stream) {
+    // the bits of `epilogue` above the low four: the activation of the gate (epilogue 1)
+    SkinnyFusion fu = fusion;
+    fu.gate_kind = epilogue >> 4;
+    epilogue &= 15;
+    FL_CHECK(fu.gate_kind >= 0 && fu.gate_kind <= FL_GATE_GELU_ERF && (fu.gate_kind == 0 || epilogue == EPI_SWIGLU),
+             "gemm_skinny: gate activation %d with epilogue %d", fu.gate_kind, epilogue);
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(M <= 64, "gemm_skinny: %d rows, at most 64", M);
     {
@@ -490,7 +497,7 @@ static int skinny_entry(const void* x, const void* w_packed, void* out, int out_
 // out[M, out_cols] = silu(gate) * up with out_cols <= N / 2.
 extern "C" int fl_gemm_skinny(const void* x, const void* w_packed, void* out, int out_dtype, int M, int N,
                               int K, int nw_hint, int epilogue, int out_cols, hipStream_t stream) {
-    FL_CHECK(epilogue == 0 || epilogue == 1, "gemm_skinny: unknown epilogue %d", epilogue);
+    FL_CHECK((epilogue & 15) == 0 || (epilogue & 15) == 1, "gemm_skinny: unknown epilogue %d", epilogue);
     const SkinnyFusion none = {nullptr, 0, 0.f, nullptr, nullptr, nullptr, nullptr};
     return skinny_entry(x, w_packed, out, out_dtype, M, N, K, nw_hint, epilogue, out_cols, none, RopeStore{}, stream);
 }

@@ -52,6 +52,7 @@ struct TiledFusion {
     const float* g;
     bf16_t* xg;
     float* out_ssq;
+    int gate_kind;             // the SwiGLU epilogue's activation of the gate (FL_GATE_*, 0 = silu)
 };
 
 
@@ -335,7 +336,7 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const float gv = acc[ta][tb][r];
-                        act[r] = gv / (1.0f + expf(-gv)) * up[r];
+                        act[r] = gate_activation(gv, fu.gate_kind) * up[r];
                     }
                     TOut* p = out + (size_t)tok * out_cols + f0;
                     if (out_cols % 4 == 0 && f0 + 4 <= out_cols) {
@@ -513,7 +514,10 @@ extern "C" int fl_gemm_tiled_ex(const void* x, const void* w_packed, void* out, 
     FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled: bad sizes M=%d N=%d K=%d", M, N, K);
     FL_CHECK(K % 8 == 0, "gemm_tiled: K=%d is no multiple of 8 (16-byte loads)", K);
     FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "gemm_tiled: unknown output dtype %d", out_dtype);
+    const int gate_kind = epilogue >> 4;          // the bits above the low four: the activation of the gate (epilogue 1)
+    epilogue &= 15;
     FL_CHECK(epilogue == 0 || epilogue == 1, "gemm_tiled: unknown epilogue %d", epilogue);
+    FL_CHECK(gate_kind >= 0 && gate_kind <= FL_GATE_GELU_ERF && (gate_kind == 0 || epilogue == 1), "gemm_tiled: gate activation %d", gate_kind);
     FL_CHECK(epilogue == 0 ? out_cols == N : (N % 16 == 0 && out_cols > 0 && out_cols <= N / 2),
              "gemm_tiled: %d output columns do not fit %d rows of w", out_cols, N);
     FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)out % 16 == 0),
@@ -529,7 +533,7 @@ extern "C" int fl_gemm_tiled_ex(const void* x, const void* w_packed, void* out, 
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w_packed;
     const RopeStore none{};
-    const TiledFusion fu = {in_ssq, in_parts, eps, nullptr, nullptr, nullptr, nullptr};
+    const TiledFusion fu = {in_ssq, in_parts, eps, nullptr, nullptr, nullptr, nullptr, gate_kind};
     if (epilogue) {
         if (out_dtype == FL_F32)
             launch_tiled<float, TG_SWIGLU>(v, 1, stream, xb, wb, (float*)out, M, N, K, n_steps, per, out_cols, none, fu);

@@ -130,12 +130,13 @@ class Runtime:
         from ..kernels import tuned
         return tuned.gemm_add_norm(self, x, w, resid, norm_weight, eps)
 
-    def gemm_swiglu(self, x, w, out):
-        """``out = silu(x Wg^T) * (x Wu^T)``; ``w`` comes from ``prepare_gate_up``.  The tuned
-        kernels apply the gate before they store; the plain path is a product and a gate kernel."""
+    def gemm_swiglu(self, x, w, out, gate: str = "silu"):
+        """``out = act(x Wg^T) * (x Wu^T)``, act = ``gate`` (``silu``, ``gelu_tanh`` or ``gelu``); ``w`` comes
+        from ``prepare_gate_up``.  The tuned kernels apply the gate before they store; the plain path is a
+        product and a gate kernel."""
         if self.tuned:
             from ..kernels import tuned
-            return tuned.gemm_swiglu(x, w, out, self)
+            return tuned.gemm_swiglu(x, w, out, self, gate=gate)
         gu = self.buffer("ffn_gate_up", x.shape[0], w.rows, torch.float32)
         ops.gemm_plain(x, w.rowmajor, gu)
-        return ops.silu_mul(gu, out)
+        return ops.silu_mul(gu, out) if gate == "silu" else ops.gated_act(gu, out, gate)

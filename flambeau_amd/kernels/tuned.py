@@ -116,7 +116,17 @@ def _row_scale_args(row_scale, M, K):
     return _check(row_scale.ssq, "gemm.row_scale", torch.float32, (M, parts)), parts, float(row_scale.eps)
 
 
-def gemm_skinny(x, w_packed, out, waves_per_block: int = 0, swiglu_rows: int = 0, row_scale: NormedRows | None = None):
+GATES = {"silu": 0, "gelu_tanh": 1, "gelu": 2}     # the gate's activation in the fused epilogue (FL_GATE_* of common.h)
+
+
+def _gated(gate: str) -> int:
+    """The ``epilogue`` argument of a product that applies ``act(gate) * up`` before it stores: 1, with the
+    activation's code in the bits above the low four."""
+    return 1 | (GATES[gate] << 4)
+
+
+def gemm_skinny(x, w_packed, out, waves_per_block: int = 0, swiglu_rows: int = 0, row_scale: NormedRows | None = None,
+                gate: str = "silu"):
     """``out = x @ w.T`` for up to 64 rows of x; ``w_packed`` = ``pack_weight(w)``, N rows taken
     from ``out``.  With ``swiglu_rows`` the packed matrix holds that many interleaved gate/up
     rows and ``out`` receives ``silu(gate) * up``.  With ``row_scale`` (then ``x`` is its ``xg``,
@@ -128,11 +138,11 @@ def gemm_skinny(x, w_packed, out, waves_per_block: int = 0, swiglu_rows: int = 0
     if row_scale is None:
         call("fl_gemm_skinny", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
              _check(out, "gemm.out", None, (M, None)), dtype_code(out.dtype), M, N, K, int(waves_per_block),
-             1 if swiglu_rows else 0, out.shape[1], stream_handle())
+             _gated(gate) if swiglu_rows else 0, out.shape[1], stream_handle())
         return out
     ssq, parts, eps = _row_scale_args(row_scale, M, K)
     call("fl_gemm_skinny_fused", _check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
-         _check(out, "gemm.out", None, (M, None)), dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0,
+         _check(out, "gemm.out", None, (M, None)), dtype_code(out.dtype), M, N, K, _gated(gate) if swiglu_rows else 0,
          out.shape[1], ssq, parts, eps, None, None, None, None, stream_handle())
     return out
 
@@ -279,7 +289,7 @@ def gemm_mid_splits(M: int, N: int, K: int, waves: int = 0, splits: int = 0) -> 
     return load().fl_gemm_mid_splits_ex(M, N, K, waves, splits)
 
 
-def gemm_mid(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale: NormedRows | None = None,
+def gemm_mid(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale: NormedRows | None = None, gate: str = "silu",
              waves: int = 0, splits: int = 0):
     """``out = x @ w.T`` for 17 to 64 rows of x (fewer are allowed) and K a multiple of 32: the
     waves of a block share x through LDS.  A narrow matrix splits K and needs ``workspace``
@@ -297,7 +307,7 @@ def gemm_mid(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale: 
     args = (_check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
             _check(out, "gemm.out", None, (M, None)),
             _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
-            dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], ssq, parts, eps)
+            dtype_code(out.dtype), M, N, K, _gated(gate) if swiglu_rows else 0, out.shape[1], ssq, parts, eps)
     if waves or splits:
         call("fl_gemm_mid_ex", *args, int(waves), int(splits), stream_handle())
     else:
@@ -348,7 +358,7 @@ def gemm_tiled_splits(M: int, N: int, K: int, splits: int = 0) -> int:
     return load().fl_gemm_tiled_splits_ex(M, N, K, splits)
 
 
-def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale: NormedRows | None = None,
+def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale: NormedRows | None = None, gate: str = "silu",
                variant: int = 0, splits: int = 0):
     """``out = x @ w.T`` for many rows of x.  A shape whose grid would not fill the chip splits K
     and needs ``workspace`` (float32, ``gemm_tiled_splits(M, N, K) * M * N`` values).  With
@@ -366,7 +376,7 @@ def gemm_tiled(x, w_packed, out, workspace=None, swiglu_rows: int = 0, row_scale
     args = (_check(x, "gemm.x", torch.bfloat16, (M, K)), _check(w_packed, "gemm.w", torch.bfloat16),
             _check(out, "gemm.out", None, (M, None)),
             _check(workspace, "gemm.workspace", torch.float32) if workspace is not None else None,
-            dtype_code(out.dtype), M, N, K, 1 if swiglu_rows else 0, out.shape[1], ssq, parts, eps)
+            dtype_code(out.dtype), M, N, K, _gated(gate) if swiglu_rows else 0, out.shape[1], ssq, parts, eps)
     if variant or splits:
         call("fl_gemm_tiled_ex", *args, int(variant), int(splits), stream_handle())
     else:
@@ -469,24 +479,25 @@ def gemm(x, w: Weight, out, rt=None):
     return ops.gemm_plain(x, w.rowmajor, out)
 
 
-def gemm_swiglu(x, w: Weight, out, rt):
-    """``out = silu(x Wg^T) * (x Wu^T)``; ``w`` comes from ``prepare_gate_up``; ``x`` may be ``NormedRows``."""
+def gemm_swiglu(x, w: Weight, out, rt, gate: str = "silu"):
+    """``out = act(x Wg^T) * (x Wu^T)``, act = ``gate`` (silu, gelu_tanh or gelu); ``w`` comes from
+    ``prepare_gate_up``; ``x`` may be ``NormedRows``."""
     x, scale = _rows_for(x, w, rt)
     M, K = x.shape
     if scale is not None and w.swiglu_cols:
         kernel = gemm_skinny if M <= FUSED_NORM_MAX_ROWS else (gemm_mid if M <= SKINNY_MAX_ROWS else gemm_tiled)
-        return kernel(x, w.packed, out, swiglu_rows=w.packed_rows, row_scale=scale)
+        return kernel(x, w.packed, out, swiglu_rows=w.packed_rows, row_scale=scale, gate=gate)
     if scale is not None:
         x = scale.materialize(rt)
     if w.packed is not None and w.swiglu_cols and x.dtype == torch.bfloat16 and K % 8 == 0:
         if SKINNY_BEST_ROWS < M <= SKINNY_MAX_ROWS and K % 32 == 0:
-            return gemm_mid(x, w.packed, out, swiglu_rows=w.packed_rows)
+            return gemm_mid(x, w.packed, out, swiglu_rows=w.packed_rows, gate=gate)
         if M <= SKINNY_MAX_ROWS:
-            return gemm_skinny(x, w.packed, out, swiglu_rows=w.packed_rows)
-        return gemm_tiled(x, w.packed, out, swiglu_rows=w.packed_rows)
+            return gemm_skinny(x, w.packed, out, swiglu_rows=w.packed_rows, gate=gate)
+        return gemm_tiled(x, w.packed, out, swiglu_rows=w.packed_rows, gate=gate)
     gu = rt.buffer("ffn_gate_up", M, w.rows, torch.float32)
     ops.gemm_plain(x, w.rowmajor, gu)
-    return ops.silu_mul(gu, out)
+    return ops.silu_mul(gu, out) if gate == "silu" else ops.gated_act(gu, out, gate)
 
 
 def prepare_weight(w: torch.Tensor) -> Weight:

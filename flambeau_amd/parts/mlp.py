@@ -35,33 +35,19 @@ class SwiGLU(FeedForward):
 
 
 @FEED_FORWARDS.register("gated_mlp")
-class GatedMlp(FeedForward):
-    """d = (act(x Wg^T) * (x Wu^T)) Wd^T with the activation as a parameter (``gelu``, ``gelu_tanh``, ``silu``).
-    Gate and up are one joined product with 32-bit results; the activation and the product of the two
-    halves are taken in 32-bit."""
-    replayable = True
+class GatedMlp(SwiGLU):
+    """d = (act(x Wg^T) * (x Wu^T)) Wd^T with the activation as a parameter (``gelu_tanh``, ``gelu``, ``silu``).
+    Gate and up are one joined product whose kernel applies the activation (in 32-bit) before it stores."""
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "gelu_tanh"):
         from ..kernels import ops
         if activation not in ops.ACTIVATIONS:
             raise ValueError(f"gated_mlp: unknown activation '{activation}'; known: {sorted(ops.ACTIVATIONS)}")
-        self.hidden_size, self.intermediate_size, self.activation = hidden_size, intermediate_size, activation
-
-    def tensors(self):
-        H, I = self.hidden_size, self.intermediate_size
-        return {"gate.weight": TensorSpec((I, H)), "up.weight": TensorSpec((I, H)),
-                "down.weight": TensorSpec((H, I))}
-
-    def bind(self, weights, rt):
-        self.rt = rt
-        self.w_gate_up = rt.prepare_weight(torch.cat([weights["gate.weight"], weights["up.weight"]], dim=0).contiguous())
-        self.w_down = rt.prepare_weight(weights["down.weight"])
+        super().__init__(hidden_size, intermediate_size)
+        self.activation = activation
 
     def forward(self, x, step):
-        from ..kernels import ops
         rt, n, I = self.rt, x.shape[0], self.intermediate_size
-        both = rt.buffer("gmlp_gate_up", n, 2 * I, torch.float32)
-        rt.gemm(x, self.w_gate_up, both)
-        act = rt.buffer("gmlp_act", n, I)
-        ops.gated_act(both, act, self.activation)
+        act = rt.buffer("ffn_act", n, I)
+        rt.gemm_swiglu(x, self.w_gate_up, act, gate=self.activation)
         return Product(act, self.w_down)
