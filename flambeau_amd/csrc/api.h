@@ -284,7 +284,7 @@ int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, int col_v, c
                    int dtype, int n, int nh, int nkv, int D, int Dv, int hdp, int page_size, int n_pages, int rot,
                    int interleaved, const float* cs, const float* qnorm_w, const float* knorm_w, int head_norm,
                    float eps, float* v_first, int vmix_mode, const float* lambda, int write_cache,
-                   hipStream_t stream);
+                   float* row_scales, hipStream_t stream);
 
 // ---- linear recurrences with a matrix state per head (linear_scan.hip) ----
 int fl_linear_scan_max_dim(void);

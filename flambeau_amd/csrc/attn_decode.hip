@@ -145,8 +145,8 @@ __global__ __launch_bounds__(256, HDP <= 128 ? 2 : 1) void attn_decode_kernel(
             const int ka = t0 + 8 * g + r, kb = ka + 4;
             float va = sa[r] * scale, vb = sb[r] * scale;
             if (softcap > 0.f) {                             // scores capped smoothly at +-softcap
-                va = softcap * tanhf(va / softcap);
-                vb = softcap * tanhf(vb / softcap);
+                va = softcap * fast_tanh(va / softcap);
+                vb = softcap * fast_tanh(vb / softcap);
             }
             sa[r] = (ka >= lo && ka <= p) ? va : -INFINITY;
             sb[r] = (kb >= lo && kb <= p) ? vb : -INFINITY;

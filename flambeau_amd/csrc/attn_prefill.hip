@@ -280,8 +280,8 @@ __global__ __launch_bounds__(256, QT * HDP <= 256 ? 2 : 1) void attn_prefill_ker
                 for (int t = 0; t < QT; ++t)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        sa[half][t][r] = cap_raw * tanhf(sa[half][t][r] * inv_cap);
-                        sb[half][t][r] = cap_raw * tanhf(sb[half][t][r] * inv_cap);
+                        sa[half][t][r] = cap_raw * fast_tanh(sa[half][t][r] * inv_cap);
+                        sb[half][t][r] = cap_raw * fast_tanh(sb[half][t][r] * inv_cap);
                     }
             }
             if (need_mask) {

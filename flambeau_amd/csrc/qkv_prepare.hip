@@ -15,6 +15,8 @@
 #include "api.h"
 #include "recordable.h"
 
+#define QKV_FEW_TOKENS 64     // up to this many tokens a block forms the projection's sums of squares for itself
+
 struct QkvPrepare {
     const float* proj; int ld; int col_q, col_k, col_v;
     const int* positions; const int* tok_seq; const int* block_table; int max_blocks;
@@ -23,7 +25,23 @@ struct QkvPrepare {
     const float* qnorm_w; const float* knorm_w; int head_norm; float eps;
     float* v_first; int vmix_mode; const float* lambda;
     int write_cache;
+    float* row_scales;          // [n][2]: 1 / rms of every token's q and k projection, made by a kernel of its own (or null)
 };
+
+// The norm over the whole projection of q and of k: 1 / sqrt(mean(x^2) + eps) of both for one token per block.
+__global__ __launch_bounds__(256) void qkv_row_scales_kernel(QkvPrepare a, int nkv) {
+    __shared__ float lds[8];
+    const float* row = a.proj + (size_t)blockIdx.x * a.ld;
+    float sq = 0.f, sk = 0.f;
+    for (int i = threadIdx.x; i < a.nh * a.D; i += 256) sq = fmaf(row[a.col_q + i], row[a.col_q + i], sq);
+    for (int i = threadIdx.x; i < nkv * a.D; i += 256) sk = fmaf(row[a.col_k + i], row[a.col_k + i], sk);
+    sq = block_sum<4>(sq, lds);
+    sk = block_sum<4>(sk, lds + 4);
+    if (threadIdx.x == 0) {
+        a.row_scales[2 * blockIdx.x] = 1.0f / sqrtf(sq / (float)(a.nh * a.D) + a.eps);
+        a.row_scales[2 * blockIdx.x + 1] = 1.0f / sqrtf(sk / (float)(nkv * a.D) + a.eps);
+    }
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __restrict__ q_out, PagedCache cache) {
@@ -32,7 +50,11 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __res
     const int nh = a.nh, nkv = cache.n_kv_heads, D = a.D, Dv = a.Dv, hdp = a.hdp;
     const float* row = a.proj + (size_t)token * a.ld;
     float inv_q = 1.f, inv_k = 1.f;
-    if (a.qnorm_w) {
+    if (a.qnorm_w && a.row_scales) {
+        inv_q = a.row_scales[2 * token];
+        inv_k = a.row_scales[2 * token + 1];
+    } else if (a.qnorm_w) {
+        // (a step of few tokens: every block sums for itself, in the same order as the kernel above, and a launch is saved)
         float sq = 0.f, sk = 0.f;
         for (int i = threadIdx.x; i < nh * D; i += 256) sq = fmaf(row[a.col_q + i], row[a.col_q + i], sq);
         for (int i = threadIdx.x; i < nkv * D; i += 256) sk = fmaf(row[a.col_k + i], row[a.col_k + i], sk);
@@ -114,7 +136,7 @@ extern "C" int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, i
                               int dtype, int n, int nh, int nkv, int D, int Dv, int hdp, int page_size, int n_pages, int rot,
                               int interleaved, const float* cs, const float* qnorm_w, const float* knorm_w, int head_norm,
                               float eps, float* v_first, int vmix_mode, const float* lambda, int write_cache,
-                              hipStream_t stream) {
+                              float* row_scales, hipStream_t stream) {
     FL_CHECK(n >= 0 && nh > 0 && nkv > 0 && D > 0 && Dv > 0 && page_size > 0, "qkv_prepare: bad sizes");
     FL_CHECK(hdp >= D && hdp >= Dv && hdp <= 256, "qkv_prepare: heads of %d and %d values stored %d wide (at most 256)", D, Dv, hdp);
     FL_CHECK(rot >= 0 && rot <= D && rot % 2 == 0, "qkv_prepare: rotated dims %d of head %d", rot, D);
@@ -125,10 +147,16 @@ extern "C" int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, i
              "qkv_prepare: value blending %d without its buffers", vmix_mode);
     if (n == 0) return 0;
     QkvPrepare a{proj, ld, col_q, col_k, col_v, positions, tok_seq, block_table, max_blocks, nh, D, Dv, hdp,
-                 rot, interleaved, (const float2*)cs, qnorm_w, knorm_w, head_norm, eps, v_first, vmix_mode, lambda, write_cache};
+                 rot, interleaved, (const float2*)cs, qnorm_w, knorm_w, head_norm, eps, v_first, vmix_mode, lambda, write_cache,
+                 (qnorm_w && n > QKV_FEW_TOKENS) ? row_scales : nullptr};
     PagedCache c{cache_base, nkv, page_size, hdp, n_pages};
     dim3 grid(n, ceil_div(nh + nkv, 4));
     FL_CHECK(grid.y <= 65535, "qkv_prepare: %d heads are more than one grid takes", nh + nkv);
+    if (a.row_scales) {
+        // many tokens: the sums of squares once per token, not once per block of four heads
+        qkv_row_scales_kernel<<<n, 256, 0, stream>>>(a, nkv);
+        FL_LAUNCH_CHECK();
+    }
     if (dtype == FL_F32)
         qkv_prepare_kernel<float><<<grid, 256, 0, stream>>>(a, (float*)q_out, c);
     else if (dtype == FL_BF16)

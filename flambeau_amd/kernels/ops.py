@@ -559,12 +559,14 @@ def heads_gate(x, head_stride, gate, gate_col0, kind, out, n_heads):
 
 
 def qkv_prepare(proj, cols, positions, tok_seq, block_table, q_out, cache: PagedLayerCache, n_heads, dim, vdim, rotated_dims,
-                interleaved, table, q_gain, k_gain, head_norm, eps, v_first=None, value_mix: int = 0, mix=None, write_cache=True):
+                interleaved, table, q_gain, k_gain, head_norm, eps, v_first=None, value_mix: int = 0, mix=None, write_cache=True,
+                row_scales=None):
     """From the float32 rows of a joined projection (q, k, v at the columns ``cols``) to the rotated, normed
     queries in ``q_out`` and the token's keys and values in the cache, heads stored ``cache.head_dim`` wide.
     ``q_gain`` / ``k_gain``: gains of a norm over the whole projection of q and of k (before rotation);
     ``head_norm``: every head divided by its root mean square after rotation; ``value_mix``: 1 keeps the
-    values in ``v_first``, 2 blends them with it by the device scalar ``mix``."""
+    values in ``v_first``, 2 blends them with it by the device scalar ``mix``; ``row_scales``: float32 ``[n, 2]`` of
+    scratch for the norm over the projection (a step of many tokens forms its sums in a kernel of their own)."""
     n, ld = proj.shape
     nkv, hdp = cache.n_kv_heads, cache.head_dim
     dt = cache.pool.dtype
@@ -579,7 +581,8 @@ def qkv_prepare(proj, cols, positions, tok_seq, block_table, q_out, cache: Paged
          _check(k_gain, "qkv_prepare.k_gain", torch.float32, (nkv * dim,)) if k_gain is not None else None,
          int(bool(head_norm)), float(eps),
          _check(v_first, "qkv_prepare.v_first", torch.float32, (n, nkv * vdim)) if v_first is not None else None, int(value_mix),
-         _check(mix, "qkv_prepare.mix", torch.float32) if mix is not None else None, int(bool(write_cache)), stream_handle())
+         _check(mix, "qkv_prepare.mix", torch.float32) if mix is not None else None, int(bool(write_cache)),
+         _check(row_scales, "qkv_prepare.row_scales", torch.float32, (n, 2)) if row_scales is not None else None, stream_handle())
     return q_out
 
 

@@ -211,7 +211,8 @@ class NormedGQAAttention(PagedGQAAttention):
         q = rt.buffer("nattn_q", n, H * P)
         ops.qkv_prepare(proj, self.cols, step.positions, step.tok_seq, table, q, cache.kv, H, D, Dv, self.rotated_dims,
                         self.interleaved, angles, self.q_gain, self.k_gain, self.qk_norm == "head", self.eps,
-                        v_first=v_first, value_mix=mode, mix=self.mix, write_cache=cache.writes)
+                        v_first=v_first, value_mix=mode, mix=self.mix, write_cache=cache.writes,
+                        row_scales=rt.buffer("nattn_row_scales", n, 2, torch.float32) if self.qk_norm == "projection" else None)
         out = rt.buffer("nattn_out", n, H * P)
         self.kernels.attention(q, out, cache.kv, step, table, H, self.scale, self.window, softcap=self.softcap)
         if self.gate is not None or P != Dv:
