@@ -30,10 +30,8 @@ def _position(rot, dim: int, layout: str) -> PartSpec:
         return PartSpec("none", {})
     params = dict(head_dim=dim, theta=rot.base, rotated_dims=rot.dims)
     if rot.scaling is not None:
-        if layout != "half":
-            raise ValueError("a stretched ladder of frequencies comes with the split-half rotation only")
         sc = rot.scaling
-        return PartSpec("rope_blended", dict(params, factor=sc.factor, original=sc.original, fast=sc.fast, slow=sc.slow))
+        return PartSpec("rope_blended", dict(params, factor=sc.factor, original=sc.original, fast=sc.fast, slow=sc.slow, layout=layout))
     return PartSpec("rope_neox" if layout == "half" else "rope_interleaved", params)
 
 

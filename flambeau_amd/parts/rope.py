@@ -113,13 +113,20 @@ def blended_frequencies(rotated_dims: int, theta: float, factor: float, original
 
 @POSITION_ENCODINGS.register("rope_blended")
 class RotaryBlended(RotaryNeoX):
-    """Split-half rotation with the stretched ladder of ``blended_frequencies``."""
+    """Rotation with the stretched ladder of ``blended_frequencies``; ``layout``: ``half`` (split halves, which
+    the fused rotate-and-store kernels take too) or ``interleaved``."""
 
     def __init__(self, head_dim: int, theta: float, factor: float, original: int, fast: float, slow: float,
-                 rotated_dims: int | None = None):
+                 rotated_dims: int | None = None, layout: str = "half"):
         super().__init__(head_dim, theta, rotated_dims)
+        if layout not in ("half", "interleaved"):
+            raise ValueError(f"rope_blended: layout must be 'half' or 'interleaved', got {layout!r}")
+        self.layout = layout
         self._freqs, self.magnitude = blended_frequencies(self.rotated_dims, self.theta, float(factor), int(original),
                                                            float(fast), float(slow))
 
     def inverse_frequencies(self):
         return self._freqs
+
+    def rotary_parameters(self):
+        return super().rotary_parameters() if self.layout == "half" else None

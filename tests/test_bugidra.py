@@ -176,3 +176,20 @@ def test_rotations_written_out():
     assert np.allclose(inter[:4], [1 * np.cos(a[0]) - 2 * np.sin(a[0]), 2 * np.cos(a[0]) + 1 * np.sin(a[0]),
                                    3 * np.cos(a[1]) - 4 * np.sin(a[1]), 4 * np.cos(a[1]) + 3 * np.sin(a[1])])
     assert np.array_equal(half[4:], x[0, 0, 4:]) and np.array_equal(inter[4:], x[0, 0, 4:])
+
+
+def test_a_stretched_ladder_on_either_rotation():
+    """The frequencies' stretch is a key of a rotation, whichever mixer has it: the interleaved rotation of an
+    attention layer and the retention's take it like the pair's left side."""
+    from flambeau_amd.registry import config_from_dict
+    raw = json.loads(json.dumps(CONFIGS["A"]["config"]))
+    raw["layers"][0]["mixer"]["rot"]["scaling"] = {"factor": 2.0, "original": 32, "fast": 8.0, "slow": 1.0}
+    raw["layers"][2]["mixer"]["right"]["rot"]["scaling"] = {"factor": 3.0, "original": 16, "fast": 4.0, "slow": 0.5}
+    arch, cfg = config_from_dict(raw, "test")
+    spec = arch.build_spec(cfg)
+    first = spec.layers[0].block.params["mixer"].params["position"]
+    assert first.kind == "rope_blended" and first.params["layout"] == "interleaved" and first.params["factor"] == 2.0
+    right = spec.layers[2].block.params["mixer"].params["right"].params["position"]
+    assert right.kind == "rope_blended" and right.params["layout"] == "half" and right.params["original"] == 16
+    plain = spec.layers[3].block.params["mixer"].params["position"]
+    assert plain.kind == "rope_interleaved" and plain.params["rotated_dims"] == 24

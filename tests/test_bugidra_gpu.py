@@ -227,6 +227,41 @@ def test_rotated_attention_alone(dtype, H, G, D, Dv, rd, scaling):
         assert np.abs(got - want).max() < TOL[dtype] * np.abs(want).max(), cuts
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("D,Dv,window", [(16, 24, 13), (64, 64, 70), (32, 16, 64), (24, 8, 1)])
+def test_attention_with_a_window(dtype, D, Dv, window):
+    """``window`` keys, the query's own included (no model of the package sets it for this mixer yet), with the
+    stretched ladder in the interleaved layout: against the formula written out, whole and in portions that
+    cross the window's edge and the kernels' chunks of 64 keys."""
+    from flambeau_amd.parts import MIXERS, PartSpec
+    rt = make_rt(dtype)
+    W, n, eps, H, G, scale, cap = 40, 150, 1e-5, 4, 2, 0.7, 8.0
+    scaling = (4.0, 32, 8.0, 1.0)
+    position = PartSpec("rope_blended", dict(head_dim=D, theta=900.0, rotated_dims=8, factor=scaling[0], original=scaling[1],
+                                             fast=scaling[2], slow=scaling[3], layout="interleaved"))
+    mixer, plain = bound_part(MIXERS, PartSpec("normed_gqa_attention", dict(
+        hidden_size=W, n_heads=H, n_kv_heads=G, head_dim=D, value_dim=Dv, scale=scale, position=position, qk_norm="projection",
+        eps=eps, softcap=cap, gate="silu", window=window)), dtype, rt, seed=D)
+    assert mixer.cache_spec().window == window
+    x = _x(n, W, dtype, 8)
+    h = x.double().numpy()
+    r = rot(900.0, 8, scaling)
+    q = pb.rotate(pb.rms_norm(h @ plain["m.q"].T, plain["m.q.norm"], eps).reshape(n, H, D), np.arange(n), r, "interleaved")
+    k = pb.rotate(pb.rms_norm(h @ plain["m.k"].T, plain["m.k.norm"], eps).reshape(n, G, D), np.arange(n), r, "interleaved")
+    v = (h @ plain["m.v"].T).reshape(n, G, Dv)
+    want = np.zeros((n, H, Dv))
+    for i in range(n):
+        lo = max(0, i - window + 1)
+        for a in range(H):
+            s = cap * np.tanh(k[lo:i + 1, a // (H // G)] @ q[i, a] * scale / cap)
+            p = np.exp(s - s.max())
+            want[i, a] = (p / p.sum()) @ v[lo:i + 1, a // (H // G)]
+    want = (want.reshape(n, H * Dv) * pb.silu(h @ plain["m.g"].T)) @ plain["m.o"].T
+    for cuts in ([150], [60, 4, 1, 1, 70, 2, 12], [1] * 30 + [120]):
+        got = run_mixer(mixer, rt, x, cuts, n_pages=60)
+        assert np.abs(got - want).max() < TOL[dtype] * np.abs(want).max(), cuts
+
+
 def test_the_stretched_ladder_written_out():
     """The frequencies of one small case by hand: dims 8, base 16, original 16, factor 4, fast 2, slow 0.5."""
     import math
