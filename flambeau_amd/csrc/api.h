@@ -248,6 +248,17 @@ int fl_attn_prefill_heads(int n_tiles, int nh, int nkv, int hd, int max_keys);  
 int fl_attn_prefill_workspace(int n_rows, int nh, int hd, int n_split, long* o_floats, long* ml_floats);
 int fl_attn_decode_workspace(int n_items, int nh, int hd, int n_split, long* o_floats, long* ml_floats);
 
+// ---- products that add to the residual stream and norm it with Dynamic Tanh in their epilogue ----
+// resid[M, N] += x w^T; xn[M, N] = bf16(tanh(alpha[0] * resid) * g + bias) (bias may be null).  fl_gemm_skinny_dyt: at
+// most 16 rows; fl_gemm_tiled_dyt: shapes whose K is not split (fl_gemm_tiled_splits(M, N, K) == 1).
+int fl_gemm_skinny_dyt(const void* x, const void* w_packed, int M, int N, int K, float* resid,
+                       const float* alpha, const float* g, const float* bias, void* xn, hipStream_t stream);
+int fl_gemm_tiled_dyt(const void* x, const void* w_packed, int M, int N, int K, float* resid,
+                      const float* alpha, const float* g, const float* bias, void* xn, hipStream_t stream);
+// the same from a product's K-splits left apart (part[splits][M][N]), as fl_reduce_residual
+int fl_reduce_dyt(const float* part, float* resid, const float* alpha, const float* g, const float* bias, void* xn,
+                  int M, int N, int splits, hipStream_t stream);
+
 // ---- the same attention kernels with capped scores: score <- softcap * tanh(score / softcap) ----
 int fl_attn_plain_capped(const void* q, void* out, const void* cache_base, int dtype,
                          const int* positions, const int* tok_seq, const int* block_table,

@@ -264,15 +264,18 @@ __global__ __launch_bounds__(256) void gemm_mid_reduce_kernel(const float* __res
 
 // The K-splits added to the residual stream: resid[m, c] += sum_s part[s][m][c] (rising s); xg[m, c] =
 // bf16(resid * g[c]); out_ssq[m, b] = sum of resid^2 over the 4096 columns of block b.  One block
-// per (4096 columns, row).
+// per (4096 columns, row).  With dyt_alpha the norm that follows is tanh(alpha resid) * g + bias, which needs
+// no statistic: xg holds the finished norm and out_ssq may be null.
 #define GM_RED_COLS 4096
 __global__ __launch_bounds__(1024) void gemm_mid_reduce_residual_kernel(const float* __restrict__ part,
                                                                        float* __restrict__ resid,
                                                                        const float* __restrict__ g,
                                                                        bf16_t* __restrict__ xg,
                                                                        float* __restrict__ out_ssq, int M, int N,
-                                                                       int splits) {
+                                                                       int splits, const float* __restrict__ dyt_alpha,
+                                                                       const float* __restrict__ dyt_bias) {
     __shared__ float red[16];
+    const float dyt_a = dyt_alpha ? dyt_alpha[0] : 0.f;
     const int row = blockIdx.y, c0 = blockIdx.x * GM_RED_COLS + 4 * threadIdx.x;
     const size_t total = (size_t)M * N;
     float sq = 0.f;
@@ -284,7 +287,12 @@ __global__ __launch_bounds__(1024) void gemm_mid_reduce_residual_kernel(const fl
             const f32x4 r = *(const f32x4*)(resid + at) + s;
             const f32x4 gv = *(const f32x4*)(g + c0);
             *(f32x4*)(resid + at) = r;
-            const bf16x4 o = {(bf16_t)(r[0] * gv[0]), (bf16_t)(r[1] * gv[1]), (bf16_t)(r[2] * gv[2]), (bf16_t)(r[3] * gv[3])};
+            f32x4 xo = {r[0] * gv[0], r[1] * gv[1], r[2] * gv[2], r[3] * gv[3]};
+            if (dyt_alpha) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) xo[u] = tanhf(dyt_a * r[u]) * gv[u] + (dyt_bias ? dyt_bias[c0 + u] : 0.f);
+            }
+            const bf16x4 o = {(bf16_t)xo[0], (bf16_t)xo[1], (bf16_t)xo[2], (bf16_t)xo[3]};
             *(bf16x4*)(xg + at) = o;
             sq = (r[0] * r[0] + r[1] * r[1]) + (r[2] * r[2] + r[3] * r[3]);
         } else {
@@ -293,13 +301,14 @@ __global__ __launch_bounds__(1024) void gemm_mid_reduce_residual_kernel(const fl
                 for (int z = 1; z < splits; ++z) s += part[(size_t)z * total + at + u];
                 const float r = resid[at + u] + s;
                 resid[at + u] = r;
-                xg[at + u] = from_f32<bf16_t>(r * g[c0 + u]);
+                xg[at + u] = from_f32<bf16_t>(dyt_alpha ? tanhf(dyt_a * r) * g[c0 + u] + (dyt_bias ? dyt_bias[c0 + u] : 0.f)
+                                                        : r * g[c0 + u]);
                 sq += r * r;
             }
         }
     }
     sq = block_sum<16>(sq, red);
-    if (threadIdx.x == 0) out_ssq[(size_t)row * gridDim.x + blockIdx.x] = sq;
+    if (threadIdx.x == 0 && out_ssq) out_ssq[(size_t)row * gridDim.x + blockIdx.x] = sq;
 }
 
 #define GM_STEPS 4                       // k-steps per chunk
@@ -497,7 +506,7 @@ extern "C" int fl_gemm_mid_residual(const void* x, const void* w_packed, float* 
                                 none, stream, plan.waves);
     FL_LAUNCH_CHECK();
     dim3 grid(ceil_div(N, GM_RED_COLS), M);
-    gemm_mid_reduce_residual_kernel<<<grid, 1024, 0, stream>>>(workspace, resid, g, (bf16_t*)xg, out_ssq, M, N, splits);
+    gemm_mid_reduce_residual_kernel<<<grid, 1024, 0, stream>>>(workspace, resid, g, (bf16_t*)xg, out_ssq, M, N, splits, nullptr, nullptr);
     FL_LAUNCH_CHECK();
     return 0;
 }
@@ -516,8 +525,24 @@ extern "C" int fl_reduce_residual(const float* part, float* resid, const float* 
     FL_CHECK(M <= 65535, "reduce_residual: %d rows, at most 65535", M);
     if (M == 0) return 0;
     dim3 grid(ceil_div(N, GM_RED_COLS), M);
-    gemm_mid_reduce_residual_kernel<<<grid, 1024, 0, stream>>>(part, resid, g, (bf16_t*)xg, out_ssq, M, N, splits);
+    gemm_mid_reduce_residual_kernel<<<grid, 1024, 0, stream>>>(part, resid, g, (bf16_t*)xg, out_ssq, M, N, splits, nullptr, nullptr);
     FL_LAUNCH_CHECK();
     return 0;
 }
 FL_RECORDABLE(fl_reduce_residual)
+
+// The same with the Dynamic Tanh norm: resid += the parts' sum, xn = bf16(tanh(alpha[0] * resid) * g + bias) (bias may be null).
+extern "C" int fl_reduce_dyt(const float* part, float* resid, const float* alpha, const float* g, const float* bias, void* xn,
+                             int M, int N, int splits, hipStream_t stream) {
+    FL_CHECK(M >= 0 && N > 0 && splits >= 1, "reduce_dyt: bad sizes M=%d N=%d splits=%d", M, N, splits);
+    FL_CHECK(part && resid && alpha && g && xn, "reduce_dyt: needs part, resid, alpha, g and xn");
+    FL_CHECK(((uintptr_t)part % 16 == 0) && ((uintptr_t)resid % 16 == 0) && ((uintptr_t)g % 16 == 0) &&
+             ((uintptr_t)xn % 8 == 0), "reduce_dyt: part, resid and g must be 16-byte aligned, xn 8-byte");
+    FL_CHECK(M <= 65535, "reduce_dyt: %d rows, at most 65535", M);
+    if (M == 0) return 0;
+    dim3 grid(ceil_div(N, GM_RED_COLS), M);
+    gemm_mid_reduce_residual_kernel<<<grid, 1024, 0, stream>>>(part, resid, g, (bf16_t*)xn, nullptr, M, N, splits, alpha, bias);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_reduce_dyt)

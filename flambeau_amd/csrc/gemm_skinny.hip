@@ -54,6 +54,8 @@ struct SkinnyFusion {
     bf16_t* xg;               // epilogue 2: [M][N] bf16(resid * g)
     float* out_ssq;           // epilogue 2: [M][blocks] sum of resid^2 over the block's features
     int gate_kind;            // epilogue 1: the gate's activation (FL_GATE_*, 0 = silu)
+    const float* dyt_alpha;   // epilogue 2, or null: the norm that follows is tanh(alpha resid) * g + bias, which needs no
+    const float* dyt_bias;    //   statistic: xg holds the finished norm and no sums of squares are left (bias may be null)
 };
 
 #define SKINNY_SCALE_LOADS 4     // loads of partial sums per thread for the row scale
@@ -159,14 +161,17 @@ __global__ __launch_bounds__(T == 1 ? 1024 : 512) void gemm_skinny_kernel(const 
         }
     }
     // epilogue 2: the wave that finishes a row group fetches its part of the residual stream and of g before the loop
-    f32x4 r_in[MT], g_in = {0.f, 0.f, 0.f, 0.f};
+    f32x4 r_in[MT], g_in = {0.f, 0.f, 0.f, 0.f}, b_in = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) r_in[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
     if (EPI == EPI_RESIDUAL && MT == 1 && owner) {
         const int f0 = my_grp * 16 + 4 * g;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-            if (f0 + r < N) g_in[r] = fu.g[f0 + r];
+            if (f0 + r < N) {
+                g_in[r] = fu.g[f0 + r];
+                if (fu.dyt_bias) b_in[r] = fu.dyt_bias[f0 + r];
+            }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int tok = mt * 16 + li;
@@ -295,17 +300,25 @@ __global__ __launch_bounds__(T == 1 ? 1024 : 512) void gemm_skinny_kernel(const 
                 sq += __shfl_xor(sq, 16, 64);
                 sq += __shfl_xor(sq, 32, 64);
                 if (tok < M) {
-                    if (g == 0) fu.out_ssq[(size_t)tok * groups + my_grp] = sq;
+                    if (g == 0 && fu.out_ssq) fu.out_ssq[(size_t)tok * groups + my_grp] = sq;
                     if (f0 < N) {
                         float* pr = fu.resid + (size_t)tok * N + f0;
                         bf16_t* px = fu.xg + (size_t)tok * N + f0;
+                        f32x4 xo;
+                        if (fu.dyt_alpha) {
+                            const float a = fu.dyt_alpha[0];
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) xo[r] = tanhf(a * nr[r]) * g_in[r] + b_in[r];
+                        } else {
+                            xo = (f32x4){nr[0] * g_in[0], nr[1] * g_in[1], nr[2] * g_in[2], nr[3] * g_in[3]};
+                        }
                         if (N % 4 == 0 && f0 + 4 <= N) {
                             store4(pr, nr);
-                            store4(px, (f32x4){nr[0] * g_in[0], nr[1] * g_in[1], nr[2] * g_in[2], nr[3] * g_in[3]});
+                            store4(px, xo);
                         } else {
                             for (int r = 0; r < 4 && f0 + r < N; ++r) {
                                 pr[r] = nr[r];
-                                px[r] = from_f32<bf16_t>(nr[r] * g_in[r]);
+                                px[r] = from_f32<bf16_t>(xo[r]);
                             }
                         }
                     }
@@ -457,7 +470,7 @@ static int skinny_entry(const void* x, const void* w_packed, void* out, int out_
     FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)out % 16 == 0),
              "gemm_skinny: operands must be 16-byte aligned");
     if (epilogue == EPI_RESIDUAL) {
-        FL_CHECK(fu.resid && fu.g && fu.xg && fu.out_ssq, "gemm_skinny: the residual epilogue needs resid, g, xg and out_ssq");
+        FL_CHECK(fu.resid && fu.g && fu.xg && (fu.out_ssq || fu.dyt_alpha), "gemm_skinny: the residual epilogue needs resid, g, xg and out_ssq");
         FL_CHECK(((uintptr_t)fu.resid % 16 == 0) && ((uintptr_t)fu.xg % 8 == 0), "gemm_skinny: resid and xg must be aligned to 16 and 8 bytes");
     }
     if (epilogue == EPI_ROPE) {
@@ -519,6 +532,17 @@ extern "C" int fl_gemm_skinny_fused(const void* x, const void* w_packed, void* o
                         out_cols, fu, RopeStore{}, stream);
 }
 FL_RECORDABLE(fl_gemm_skinny_fused)
+
+// resid[M, N] += x w^T, and the Dynamic Tanh norm of the sum in the same epilogue: xn[M, N] =
+// bf16(tanh(alpha[0] * resid) * g + bias) (bias may be null).  That norm takes no statistic of a row, so the
+// finished rows leave the product's kernel and the product that follows reads them as they are.
+extern "C" int fl_gemm_skinny_dyt(const void* x, const void* w_packed, int M, int N, int K, float* resid,
+                                  const float* alpha, const float* g, const float* bias, void* xn, hipStream_t stream) {
+    FL_CHECK(alpha, "gemm_skinny_dyt: needs alpha");
+    const SkinnyFusion fu = {nullptr, 0, 0.f, resid, g, (bf16_t*)xn, nullptr, 0, alpha, bias};
+    return skinny_entry(x, w_packed, resid, FL_F32, M, N, K, 0, EPI_RESIDUAL, N, fu, RopeStore{}, stream);
+}
+FL_RECORDABLE(fl_gemm_skinny_dyt)
 
 // The joined q/k/v projection of at most 16 rows with its rows in paired order: q is rotated and
 // written to q_out[M, nh * hd], k rotated and v as it is into the cache pages at the tokens'

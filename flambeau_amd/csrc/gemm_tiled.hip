@@ -53,6 +53,8 @@ struct TiledFusion {
     bf16_t* xg;
     float* out_ssq;
     int gate_kind;             // the SwiGLU epilogue's activation of the gate (FL_GATE_*, 0 = silu)
+    const float* dyt_alpha;    // the residual epilogue, or null: the norm that follows is tanh(alpha resid) * g + bias, which
+    const float* dyt_bias;     //   needs no statistic: xg holds the finished norm, out_ssq may be null (bias may be null)
 };
 
 
@@ -263,6 +265,7 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
         f32x4 gain[FT];                                               // the norm's weights of this lane's features
 #pragma unroll
         for (int ta = 0; ta < FT; ++ta) gain[ta] = *(const f32x4*)(fu.g + min(n0 + (wf * FT + ta) * 16 + 4 * g, N - 4));
+        const float dyt_a = fu.dyt_alpha ? fu.dyt_alpha[0] : 0.f;
         __syncthreads();                                              // the ring is no longer read
 #pragma unroll
         for (int tb = 0; tb < TT; ++tb) {
@@ -282,7 +285,13 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
                     const f32x4 nr = old[ta] + acc[ta][tb];
                     const f32x4 gv = gain[ta];
                     *(f32x4*)(fu.resid + (size_t)tok * N + f0) = nr;
-                    const bf16x4 o = {(bf16_t)(nr[0] * gv[0]), (bf16_t)(nr[1] * gv[1]), (bf16_t)(nr[2] * gv[2]), (bf16_t)(nr[3] * gv[3])};
+                    f32x4 xo = {nr[0] * gv[0], nr[1] * gv[1], nr[2] * gv[2], nr[3] * gv[3]};
+                    if (fu.dyt_alpha) {
+                        const f32x4 bv = fu.dyt_bias ? *(const f32x4*)(fu.dyt_bias + f0) : (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) xo[r] = tanhf(dyt_a * nr[r]) * gv[r] + bv[r];
+                    }
+                    const bf16x4 o = {(bf16_t)xo[0], (bf16_t)xo[1], (bf16_t)xo[2], (bf16_t)xo[3]};
                     *(bf16x4*)(fu.xg + (size_t)tok * N + f0) = o;
                     sq += (nr[0] * nr[0] + nr[1] * nr[1]) + (nr[2] * nr[2] + nr[3] * nr[3]);
                 }
@@ -293,7 +302,7 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
         }
         __syncthreads();
         for (int t = tid; t < NTT * 16; t += NW * 64)
-            if (m0 + t < M) fu.out_ssq[(size_t)(m0 + t) * n_ft + tile_f] = s_part[t] + s_part[NTT * 16 + t];
+            if (m0 + t < M && fu.out_ssq) fu.out_ssq[(size_t)(m0 + t) * n_ft + tile_f] = s_part[t] + s_part[NTT * 16 + t];
         return;
     }
     if (EPI == TG_ROPE) {
@@ -605,6 +614,29 @@ extern "C" int fl_gemm_tiled_residual_ex(const void* x, const void* w_packed, fl
     return 0;
 }
 FL_RECORDABLE(fl_gemm_tiled_residual_ex)
+
+// resid[M, N] += x w^T with the Dynamic Tanh norm of the sum in the same epilogue, xn = bf16(tanh(alpha[0] * resid)
+// * g + bias), as fl_gemm_skinny_dyt; for shapes whose K the plan does not split (fl_gemm_tiled_splits(M, N, K) == 1).
+extern "C" int fl_gemm_tiled_dyt(const void* x, const void* w_packed, int M, int N, int K, float* resid,
+                                 const float* alpha, const float* g, const float* bias, void* xn, hipStream_t stream) {
+    FL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled_dyt: bad sizes M=%d N=%d K=%d", M, N, K);
+    FL_CHECK(K % 8 == 0, "gemm_tiled_dyt: K=%d is no multiple of 8 (16-byte loads)", K);
+    FL_CHECK(N % 4 == 0, "gemm_tiled_dyt: N=%d is no multiple of 4 (16-byte accesses to the residual rows)", N);
+    FL_CHECK(resid && alpha && g && xn, "gemm_tiled_dyt: needs resid, alpha, g and xn");
+    FL_CHECK(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_packed % 16 == 0) && ((uintptr_t)resid % 16 == 0) &&
+             ((uintptr_t)g % 16 == 0) && (!bias || (uintptr_t)bias % 16 == 0) && ((uintptr_t)xn % 8 == 0),
+             "gemm_tiled_dyt: operands must be aligned (16 bytes, xn 8)");
+    if (M == 0) return 0;
+    const int n_steps = ceil_div(K, 32);
+    const TilePlan plan = tiled_plan(M, N, K, true, 0, 0);
+    FL_CHECK(plan.splits == 1, "gemm_tiled_dyt: this shape splits K %d ways; run product and norm apart", plan.splits);
+    const TiledFusion fu = {nullptr, 0, 0.f, resid, g, (bf16_t*)xn, nullptr, 0, alpha, bias};
+    launch_tiled<float, TG_RESIDUAL>(plan.variant, 1, stream, (const bf16_t*)x, (const bf16_t*)w_packed, resid, M, N, K,
+                                     n_steps, n_steps, N, RopeStore{}, fu);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_gemm_tiled_dyt)
 
 extern "C" int fl_gemm_tiled_residual(const void* x, const void* w_packed, float* workspace, int M, int N, int K,
                                       float* resid, const float* g, void* xg, float* out_ssq, hipStream_t stream) {

@@ -130,6 +130,14 @@ class Runtime:
         from ..kernels import tuned
         return tuned.gemm_add_norm(self, x, w, resid, norm_weight, eps)
 
+    def gemm_add_dyt(self, x, w, resid, alpha, gain, bias):
+        """``resid += x @ w.T`` with the Dynamic Tanh norm that follows computed by the same kernel
+        (``kernels.tuned.gemm_add_dyt``): the normed rows, or ``None`` if no kernel does both."""
+        if not self.tuned:
+            return None
+        from ..kernels import tuned
+        return tuned.gemm_add_dyt(self, x, w, resid, alpha, gain, bias)
+
     def gemm_swiglu(self, x, w, out, gate: str = "silu"):
         """``out = act(x Wg^T) * (x Wu^T)``, act = ``gate`` (``silu``, ``gelu_tanh`` or ``gelu``); ``w`` comes
         from ``prepare_gate_up``.  The tuned kernels apply the gate before they store; the plain path is a

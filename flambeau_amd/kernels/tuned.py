@@ -45,6 +45,9 @@ register_signatures({
     "fl_attn_prefill_takes": [I, I, I, I],
     "fl_attn_decode": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, P],
     "fl_attn_decode_items": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, P, I, P],
+    "fl_gemm_skinny_dyt": [P, P, I, I, I, P, P, P, P, P, P],
+    "fl_gemm_tiled_dyt": [P, P, I, I, I, P, P, P, P, P, P],
+    "fl_reduce_dyt": [P, P, P, P, P, P, I, I, I, P],
     "fl_attn_decode_items_capped": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, F, P, I, P],
     "fl_attn_prefill_capped": [P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, F, I, P, P, I, P],
 })
@@ -282,6 +285,45 @@ def gemm_add_norm(rt, x, w: Weight, resid, norm_weight, eps: float):
         workspace = _split_workspace(rt, splits * n * H, x.device) if splits > 1 else None
         return gemm_tiled_residual(x, w.packed, resid, norm_weight, xg, ssq, eps, workspace)
     return None
+
+
+def gemm_add_dyt(rt, x, w: Weight, resid, alpha, gain, bias):
+    """``resid += x @ w.T`` and the Dynamic Tanh norm of the sum, ``tanh(alpha * resid) * gain + bias`` in the
+    compute dtype, by the product's own kernel: that norm takes no statistic of a row, so nothing is left in
+    factors and the finished rows are returned.  ``None`` where no kernel takes the shape (the rows between
+    the skinny and the tiled kernel, a K that is split, sizes out of step): the caller then runs product and
+    norm apart."""
+    n, H = resid.shape
+    if (w.packed is None or w.swiglu_cols or isinstance(x, NormedRows) or x.dtype != torch.bfloat16
+            or x.shape[1] % 8 or H % 8):
+        return None
+    K = x.shape[1]
+    if w.packed.numel() != _packed_size(H, K):
+        return None
+    xn = rt.buffer("normed_dyt", n, H)
+    tail = (_check(resid, "gemm.resid", torch.float32, (n, H)), _check(alpha, "gemm.alpha", torch.float32),
+            _check(gain, "gemm.gain", torch.float32, (H,)), _check(bias, "gemm.bias", torch.float32, (H,)) if bias is not None else None,
+            _check(xn, "gemm.xn", torch.bfloat16, (n, H)))
+    parts = None
+    if n <= FUSED_NORM_MAX_ROWS and not (H % 32 == 0 and mid_preferred(n, H, K)):
+        name = "fl_gemm_skinny_dyt"
+    elif n <= SKINNY_MAX_ROWS:
+        # 17 to 64 rows: the kernel that adds the K-splits of the product does it
+        if K % 32 or H % 32:
+            return None
+        workspace = _split_workspace(rt, gemm_mid_splits(n, H, K) * n * H, x.device)
+        parts = gemm_mid_partials(x, w.packed, workspace, H)
+    elif gemm_tiled_splits(n, H, K) == 1:
+        name = "fl_gemm_tiled_dyt"
+    else:
+        workspace = _split_workspace(rt, gemm_tiled_splits(n, H, K) * n * H, x.device)
+        parts = gemm_tiled_partials(x, w.packed, workspace, H)
+    if parts is not None:
+        call("fl_reduce_dyt", _check(parts, "gemm.parts", torch.float32, (None, n, H)), *tail, n, H, parts.shape[0], stream_handle())
+    else:
+        call(name, _check(x, "gemm.x", torch.bfloat16, (n, K)), _check(w.packed, "gemm.w", torch.bfloat16), n, H, K, *tail,
+             stream_handle())
+    return xn
 
 
 def gemm_mid_splits(M: int, N: int, K: int, waves: int = 0, splits: int = 0) -> int:

@@ -129,7 +129,7 @@ class NormedGQAAttention(PagedGQAAttention):
     One joined product gives q, k, v and the gate's logits in 32-bit; norms, rotation and the blend are
     32-bit; this step's keys are stored before attention runs."""
     graph_safe = True
-    lazy_input = False
+    lazy_input = True        # its input goes to the joined projection only
     replayable = True
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PartSpec,

@@ -27,6 +27,7 @@ from .base import MIXERS, POSITION_ENCODINGS, Mixer, PartSpec, Product, StateSpe
 class Retention(Mixer):
     graph_safe = False          # a step run twice advances the state twice
     replayable = True
+    lazy_input = True           # its input goes to the joined projection only
 
     def __init__(self, hidden_size: int, n_heads: int, head_dim: int, value_dim: int, decay, position: PartSpec, eps: float,
                  key_scale: float | None = None, gate: str | None = "silu"):
@@ -94,6 +95,7 @@ class Retention(Mixer):
 class GatedDelta(Mixer):
     graph_safe = False
     replayable = True
+    lazy_input = True
 
     def __init__(self, hidden_size: int, n_heads: int, n_qk_heads: int, head_dim: int, value_dim: int, conv_taps: int, eps: float,
                  unit_eps: float = 1e-6, query_scale: float | None = None):

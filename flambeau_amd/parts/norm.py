@@ -60,3 +60,9 @@ class DynamicTanh(Norm):
 
     def forward(self, x, out, delta=None, store_sum=False, rows=None):
         return ops.dyt(x, self.alpha, self.weight, self.bias, out, delta=delta, store_sum=store_sum, rows=rows)
+
+    def after_product(self, rt, resid, product):
+        """Where a kernel for the shape exists the product's kernel adds its result to the stream and norms the
+        sum in its epilogue (nothing crosses the values of a row, so the norm is finished there): the normed
+        rows come back as a tensor and no norm kernel runs."""
+        return rt.gemm_add_dyt(product.x, product.weight, resid, self.alpha, self.weight, self.bias)

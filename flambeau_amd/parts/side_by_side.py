@@ -15,6 +15,10 @@ class SideBySide(Mixer):
     replayable = True
     graph_safe = True           # as far as it goes itself: its members are asked one by one (``mixers``)
 
+    @property
+    def lazy_input(self):
+        return all(m.lazy_input for m in self._members.values())
+
     def __init__(self, hidden_size: int, left: PartSpec, right: PartSpec, eps: float, factors=(0.5, 0.5)):
         self.hidden_size, self.eps = hidden_size, float(eps)
         self.factors = (float(factors[0]), float(factors[1]))

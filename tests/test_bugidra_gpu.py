@@ -154,6 +154,38 @@ def test_dynamic_tanh_and_scaled_embedding(dtype):
     assert torch.equal(got.cpu(), table[toks.cpu().long()].float() * 7.25)
 
 
+@pytest.mark.parametrize("n,K,H", [(1, 256, 128), (8, 512, 192), (16, 64, 4096), (40, 256, 128), (100, 256, 128), (300, 1024, 512), (700, 128, 96), (512, 512, 2048)])
+def test_a_product_that_norms_in_its_epilogue(n, K, H):
+    """The product that adds to the stream and applies Dynamic Tanh before it stores (few rows: the skinny
+    kernel, many: the tiled one) against product, addition and norm apart."""
+    from flambeau_amd.kernels import ops, tuned
+    from flambeau_amd.parts import NORMS, PartSpec, Product, ResidualStream
+    rt = make_rt("bfloat16", max_tokens=1024)
+    norm, plain = bound_part(NORMS, PartSpec("dynamic_tanh", dict(hidden_size=H)), "bfloat16", rt, seed=n, prefix="n.")
+    gen = torch.Generator().manual_seed(K)
+    x = (torch.randn(n, K, generator=gen) * 0.5).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(H, K, generator=gen) * 0.1).to(torch.bfloat16).to(DEV)
+    resid0 = torch.randn(n, H, generator=gen).to(DEV)
+    weight = rt.prepare_weight(w)
+    resid = resid0.clone()
+    fused = tuned.gemm_add_dyt(rt, x, weight, resid, norm.alpha, norm.weight, norm.bias)
+    want_resid = resid0.double() + x.double() @ w.double().T
+    if fused is None:
+        # a shape whose K the tiled product splits, or rows between the two kernels: product and norm run apart
+        assert 16 < n <= 64 or tuned.gemm_tiled_splits(n, H, K) > 1
+        stream = ResidualStream(resid0.clone(), rt)
+        stream.push(Product(x, weight))
+        fused, resid = stream.normed(norm, lazy=True), stream.resid
+    assert (resid.double() - want_resid).abs().max().item() < 2e-4 * want_resid.abs().max().item()
+    want = pb.dynamic_tanh(want_resid.cpu().numpy(), plain, "n")
+    assert np.abs(fused.double().cpu().numpy() - want).max() < 1e-2 * np.abs(want).max()
+    # and through the stream, as a block does it
+    stream = ResidualStream(resid0.clone(), rt)
+    stream.push(Product(x, weight))
+    via = stream.normed(norm, lazy=True).clone()
+    assert stream.pending is None and torch.equal(via, fused) and torch.equal(stream.resid, resid)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("W,F", [(40, 24), (36, 50), (64, 128)])
 def test_gated_feed_forward(dtype, W, F):
