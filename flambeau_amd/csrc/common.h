@@ -43,10 +43,19 @@ template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return
 #define FL_GATE_SILU 0
 #define FL_GATE_GELU_TANH 1
 #define FL_GATE_GELU_ERF 2
-__device__ __forceinline__ float gate_activation(float z, int kind) {
-    if (kind == FL_GATE_GELU_TANH) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
-    if (kind == FL_GATE_GELU_ERF) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+template <int KIND>
+__device__ __forceinline__ float gate_activation(float z) {
+    if (KIND == FL_GATE_GELU_TANH) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+    if (KIND == FL_GATE_GELU_ERF) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
     return z / (1.0f + expf(-z));
+}
+// f(constant of the kind): the choice is made once, outside the loops over a block's values (a branch per value
+// cost the tiled gate/up product 7 % of its time)
+template <typename F>
+__device__ __forceinline__ void with_gate_kind(int kind, F&& f) {
+    if (kind == FL_GATE_GELU_TANH) f(std::integral_constant<int, FL_GATE_GELU_TANH>{});
+    else if (kind == FL_GATE_GELU_ERF) f(std::integral_constant<int, FL_GATE_GELU_ERF>{});
+    else f(std::integral_constant<int, FL_GATE_SILU>{});
 }
 
 // tanh from one exponential and one reciprocal of the hardware: 1 - 2 / (1 + e^(2x)).  Both ends saturate to

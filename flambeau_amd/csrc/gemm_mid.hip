@@ -224,8 +224,10 @@ __global__ __launch_bounds__(GM_NW * 64) void gemm_mid_kernel(const bf16_t* x, c
             const int f0 = group * 8 + 2 * g;
             if ((g & 1) == 0 && tok < M && f0 < out_cols) {
                 f32x4 act;
+                with_gate_kind(gate_kind, [&](auto kind) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) act[r] = gate_activation(acc[mt][r], gate_kind) * up[r];
+                    for (int r = 0; r < 4; ++r) act[r] = gate_activation<decltype(kind)::value>(acc[mt][r]) * up[r];
+                });
                 TOut* p = out + (size_t)tok * out_cols + f0;
                 if (out_cols % 4 == 0 && f0 + 4 <= out_cols) {
                     gm_store4<TOut>(p, act);

@@ -330,8 +330,10 @@ __global__ __launch_bounds__(T == 1 ? 1024 : 512) void gemm_skinny_kernel(const 
                 const int f0 = my_grp * 8 + 2 * g;                                     // g even: features 8 b + 4 (g / 2)
                 if ((g & 1) == 0 && tok < M && f0 < out_cols) {
                     f32x4 act;
+                    with_gate_kind(fu.gate_kind, [&](auto kind) {
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) act[r] = gate_activation(sum[r], fu.gate_kind) * up[r];
+                        for (int r = 0; r < 4; ++r) act[r] = gate_activation<decltype(kind)::value>(sum[r]) * up[r];
+                    });
                     TOut* p = out + (size_t)tok * out_cols + f0;
                     if (out_cols % 4 == 0 && f0 + 4 <= out_cols) {
                         store4(p, act);

@@ -267,39 +267,44 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
         for (int ta = 0; ta < FT; ++ta) gain[ta] = *(const f32x4*)(fu.g + min(n0 + (wf * FT + ta) * 16 + 4 * g, N - 4));
         const float dyt_a = fu.dyt_alpha ? fu.dyt_alpha[0] : 0.f;
         __syncthreads();                                              // the ring is no longer read
+        // (which norm follows is chosen once, outside the loops: the usual form's code stays what it was)
+        auto add_and_norm = [&](auto dyt) {
 #pragma unroll
-        for (int tb = 0; tb < TT; ++tb) {
-            const int tok = m0 + (wt * TT + tb) * 16 + j;
-            float sq = 0.f;
-            f32x4 old[FT];                                            // the token's residual values, read together
+            for (int tb = 0; tb < TT; ++tb) {
+                const int tok = m0 + (wt * TT + tb) * 16 + j;
+                float sq = 0.f;
+                f32x4 old[FT];                                        // the token's residual values, read together
 #pragma unroll
-            for (int ta = 0; ta < FT; ++ta) {
-                const int f0 = min(n0 + (wf * FT + ta) * 16 + 4 * g, N - 4);
-                old[ta] = PREFETCH ? pre[PREFETCH ? ta : 0][PREFETCH ? tb : 0]
-                                   : *(const f32x4*)(fu.resid + (size_t)min(tok, M - 1) * N + f0);
-            }
-#pragma unroll
-            for (int ta = 0; ta < FT; ++ta) {
-                const int f0 = n0 + (wf * FT + ta) * 16 + 4 * g;
-                if (tok < M && f0 < N) {
-                    const f32x4 nr = old[ta] + acc[ta][tb];
-                    const f32x4 gv = gain[ta];
-                    *(f32x4*)(fu.resid + (size_t)tok * N + f0) = nr;
-                    f32x4 xo = {nr[0] * gv[0], nr[1] * gv[1], nr[2] * gv[2], nr[3] * gv[3]};
-                    if (fu.dyt_alpha) {
-                        const f32x4 bv = fu.dyt_bias ? *(const f32x4*)(fu.dyt_bias + f0) : (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) xo[r] = tanhf(dyt_a * nr[r]) * gv[r] + bv[r];
-                    }
-                    const bf16x4 o = {(bf16_t)xo[0], (bf16_t)xo[1], (bf16_t)xo[2], (bf16_t)xo[3]};
-                    *(bf16x4*)(fu.xg + (size_t)tok * N + f0) = o;
-                    sq += (nr[0] * nr[0] + nr[1] * nr[1]) + (nr[2] * nr[2] + nr[3] * nr[3]);
+                for (int ta = 0; ta < FT; ++ta) {
+                    const int f0 = min(n0 + (wf * FT + ta) * 16 + 4 * g, N - 4);
+                    old[ta] = PREFETCH ? pre[PREFETCH ? ta : 0][PREFETCH ? tb : 0]
+                                       : *(const f32x4*)(fu.resid + (size_t)min(tok, M - 1) * N + f0);
                 }
+#pragma unroll
+                for (int ta = 0; ta < FT; ++ta) {
+                    const int f0 = n0 + (wf * FT + ta) * 16 + 4 * g;
+                    if (tok < M && f0 < N) {
+                        const f32x4 nr = old[ta] + acc[ta][tb];
+                        const f32x4 gv = gain[ta];
+                        *(f32x4*)(fu.resid + (size_t)tok * N + f0) = nr;
+                        f32x4 xo = {nr[0] * gv[0], nr[1] * gv[1], nr[2] * gv[2], nr[3] * gv[3]};
+                        if (decltype(dyt)::value) {
+                            const f32x4 bv = fu.dyt_bias ? *(const f32x4*)(fu.dyt_bias + f0) : (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) xo[r] = tanhf(dyt_a * nr[r]) * gv[r] + bv[r];
+                        }
+                        const bf16x4 o = {(bf16_t)xo[0], (bf16_t)xo[1], (bf16_t)xo[2], (bf16_t)xo[3]};
+                        *(bf16x4*)(fu.xg + (size_t)tok * N + f0) = o;
+                        sq += (nr[0] * nr[0] + nr[1] * nr[1]) + (nr[2] * nr[2] + nr[3] * nr[3]);
+                    }
+                }
+                sq += __shfl_xor(sq, 16, 64);
+                sq += __shfl_xor(sq, 32, 64);
+                if (g == 0) s_part[wf * (NTT * 16) + (wt * TT + tb) * 16 + j] = sq;
             }
-            sq += __shfl_xor(sq, 16, 64);
-            sq += __shfl_xor(sq, 32, 64);
-            if (g == 0) s_part[wf * (NTT * 16) + (wt * TT + tb) * 16 + j] = sq;
-        }
+        };
+        if (fu.dyt_alpha) add_and_norm(std::true_type{});
+        else add_and_norm(std::false_type{});
         __syncthreads();
         for (int t = tid; t < NTT * 16; t += NW * 64)
             if (m0 + t < M && fu.out_ssq) fu.out_ssq[(size_t)(m0 + t) * n_ft + tile_f] = s_part[t] + s_part[NTT * 16 + t];
@@ -331,31 +336,30 @@ __global__ __launch_bounds__(128 * WT, OCC) void gemm_async_kernel(const bf16_t*
         return;
     }
     if (EPI == TG_SWIGLU) {
+        with_gate_kind(fu.gate_kind, [&](auto kind) {
 #pragma unroll
-        for (int tb = 0; tb < TT; ++tb) {
-            const int tok = m0 + (wt * TT + tb) * 16 + j;
+            for (int tb = 0; tb < TT; ++tb) {
+                const int tok = m0 + (wt * TT + tb) * 16 + j;
 #pragma unroll
-            for (int ta = 0; ta < FT; ++ta) {
-                f32x4 up;
+                for (int ta = 0; ta < FT; ++ta) {
+                    f32x4 up;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) up[r] = __shfl_down(acc[ta][tb][r], 16, 64);
-                const int f0 = (n0 >> 1) + (wf * FT + ta) * 8 + 2 * g;
-                if ((g & 1) == 0 && tok < M && f0 < out_cols) {
-                    f32x4 act;
+                    for (int r = 0; r < 4; ++r) up[r] = __shfl_down(acc[ta][tb][r], 16, 64);
+                    const int f0 = (n0 >> 1) + (wf * FT + ta) * 8 + 2 * g;
+                    if ((g & 1) == 0 && tok < M && f0 < out_cols) {
+                        f32x4 act;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float gv = acc[ta][tb][r];
-                        act[r] = gate_activation(gv, fu.gate_kind) * up[r];
-                    }
-                    TOut* p = out + (size_t)tok * out_cols + f0;
-                    if (out_cols % 4 == 0 && f0 + 4 <= out_cols) {
-                        tg_store4<TOut>(p, act);
-                    } else {
-                        for (int r = 0; r < 4 && f0 + r < out_cols; ++r) p[r] = from_f32<TOut>(act[r]);
+                        for (int r = 0; r < 4; ++r) act[r] = gate_activation<decltype(kind)::value>(acc[ta][tb][r]) * up[r];
+                        TOut* p = out + (size_t)tok * out_cols + f0;
+                        if (out_cols % 4 == 0 && f0 + 4 <= out_cols) {
+                            tg_store4<TOut>(p, act);
+                        } else {
+                            for (int r = 0; r < 4 && f0 + r < out_cols; ++r) p[r] = from_f32<TOut>(act[r]);
+                        }
                     }
                 }
             }
-        }
+        });
         return;
     }
     TOut* obase = out + (size_t)blockIdx.z * M * N;
